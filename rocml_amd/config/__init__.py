@@ -3,9 +3,10 @@ from .spec import (AttentionSpec, BlockSpec, GatedMlpSpec, LatentAttentionSpec, 
 from .qwen3 import Qwen3Config
 from .dokulix import DokulixConfig
 from .felovik import FelovikConfig
+from .sogavik import SogavikConfig
 from .registry import (Architecture, architecture, architecture_of, known_architectures,
                        read_config_json, register_architecture)
 
-__all__ = ["AttentionSpec", "BlockSpec", "GatedMlpSpec", "LatentAttentionSpec", "DokulixConfig", "FelovikConfig", "ModelSpec", "NormSpec", "RopeSpec",
+__all__ = ["AttentionSpec", "BlockSpec", "GatedMlpSpec", "LatentAttentionSpec", "DokulixConfig", "FelovikConfig", "SogavikConfig", "ModelSpec", "NormSpec", "RopeSpec",
            "ScheduleEntry", "default_schedule", "Qwen3Config", "Architecture", "architecture",
            "architecture_of", "known_architectures", "read_config_json", "register_architecture"]

@@ -118,6 +118,13 @@ def _register_builtin() -> None:
         to_spec=lambda cfg: cfg.to_model_spec(),
         checkpoint_names=felovik.checkpoint_names,
         unused_tensors=felovik.unused_tensors))
+    from . import sogavik
+    register_architecture(Architecture(
+        name=sogavik.ARCHITECTURE,
+        read_config=sogavik.SogavikConfig.from_dict,
+        to_spec=lambda cfg: cfg.to_model_spec(),
+        checkpoint_names=sogavik.checkpoint_names,
+        unused_tensors=sogavik.unused_tensors))
 
 
 _register_builtin()

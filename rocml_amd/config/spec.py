@@ -31,13 +31,37 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """Norm with a weight and a bias: ``(x - mean) / sqrt(var + eps) * weight + bias``, ``var`` the
+    mean of the squared deviations from the mean."""
+    size: int
+    eps: float
+    kind: str = "layernorm"
+
+
+@dataclass(frozen=True)
+class RopeStretch:
+    """Frequencies slowed down for contexts longer than ``original`` positions (YaRN): with
+    ``d(t) = rot_dim ln(original / (2 pi t)) / (2 ln theta)``, ``lo = max(floor(d(fast)), 0)``,
+    ``hi = min(ceil(d(slow)), rot_dim - 1)`` and ``r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``,
+    frequency ``i`` becomes ``f_i / factor * r_i + f_i (1 - r_i)``, and cosines and sines are
+    multiplied by ``0.1 ln(factor) + 1``."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Rotary position encoding with NEOX pairing ``(i, i + rot_dim/2)`` over the
-    first ``rot_dim`` values of a head; ``theta`` is the frequency base."""
+    first ``rot_dim`` values of a head; ``theta`` is the frequency base.  ``stretch``: the
+    frequencies are slowed down as ``RopeStretch`` says."""
     head_dim: int
     rot_dim: int
     theta: float
     kind: str = "rope_neox"
+    stretch: Optional[RopeStretch] = None
 
 
 @dataclass(frozen=True)
@@ -55,7 +79,12 @@ class AttentionSpec:
     query ``i`` and key ``j``.  ``sink``: the softmax's denominator has one more term, ``exp(0)``,
     which has no value.  ``q_temp``: ``(coef, every)``; the query at position ``p`` is multiplied by
     ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm.  ``gate``: the concatenated heads
-    are multiplied by ``sigmoid(W_g h)`` of the mixer's input before the output projection."""
+    are multiplied by ``sigmoid(W_g h)`` of the mixer's input before the output projection; with
+    ``gate_per_head`` the gate is one number per query head instead of one per value.
+    ``o_bias``: whether the output projection has a bias when it is not what ``bias`` says (None: as
+    ``bias``).  ``qk_norm_span``: ``"head"``, every head of q and of k is normed by itself with a gain
+    of the head's size, or ``"projection"``, a token's whole q row (all heads side by side) is
+    normed at once with a gain of that size, and its k row likewise."""
     hidden: int
     n_heads: int
     n_kv_heads: int
@@ -72,6 +101,9 @@ class AttentionSpec:
     sink: bool = False
     q_temp: Optional[Tuple[float, int]] = None
     gate: bool = False
+    gate_per_head: bool = False
+    o_bias: Optional[bool] = None
+    qk_norm_span: str = "head"
 
 
 @dataclass(frozen=True)
@@ -121,7 +153,9 @@ class RoutedExpertsSpec:
     softmax over all experts are 32-bit.  ``groups``: ``(count, keep)``; the experts form ``count``
     equal groups of neighbours, a group's score is its largest expert score, and only experts of
     the ``keep`` best groups can be chosen.  The chosen experts' scores, divided by their sum plus
-    ``sum_eps``, weight their outputs."""
+    ``sum_eps``, weight their outputs.  ``weighting`` ``"softmax_chosen"`` instead: the experts with
+    the largest logits are chosen and the weights are the softmax over the chosen logits alone (no
+    groups).  ``router_bias``: a bias vector is added to the router's logits."""
     hidden: int
     n_experts: int
     top: int
@@ -130,6 +164,8 @@ class RoutedExpertsSpec:
     groups: Optional[Tuple[int, int]] = None
     sum_eps: float = 1e-20
     kind: str = "routed_experts"
+    weighting: str = "softmax_all"
+    router_bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -151,6 +187,48 @@ class StateSpaceSpec:
     norm_groups: int
     eps: float
     kind: str = "state_space"
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A recurrence whose state per head is a matrix ``S`` (``head_dim x v_head_dim``), a vector
+    ``n`` (``head_dim``) and a running maximum ``m``, all zero when a sequence starts (the mLSTM of
+    xLSTM).  ``q = W_q h / sqrt(head_dim)``, ``k = W_k h``, ``v = W_v h``; per head a log input gate
+    ``i = cap tanh((W_i h + b_i) / cap)`` and a log forget gate
+    ``f = logsigmoid(cap tanh((W_f h + b_f) / cap))``; ``m' = max(f + m, i)``,
+    ``S' = exp(f + m - m') S + exp(i - m') k v^T``, ``n'`` the same with ``k`` alone, and the head's
+    output is ``S'^T q / (max(|n' . q|, exp(-m')) + floor)``.  Every head's output is divided by its
+    root mean square, the heads side by side are multiplied by a gain and by ``sigmoid(W_g h)`` and
+    projected back.  State and gates are 32-bit."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_head_dim: int
+    gate_cap: float
+    eps: float
+    floor: float = 1e-6
+    kind: str = "matrix_memory"
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A per-token input that depends on the token's id: with ``e`` the columns ``column0 ..
+    column0 + dim - 1`` of the token's row of the model's table ``table``, the result is
+    ``W_proj (act(W_gate x) * e)``."""
+    hidden: int
+    dim: int
+    table: str
+    column0: int
+    activation: str = "gelu_tanh"
+    kind: str = "token_side"
+
+
+@dataclass(frozen=True)
+class TableSpec:
+    """A matrix ``[rows, cols]`` of the model that several layers read (each its own columns)."""
+    name: str
+    rows: int
+    cols: int
 
 
 @dataclass(frozen=True)
@@ -205,13 +283,18 @@ class BlockSpec:
     ``x += mixer(norm(x)); x += ffn(norm(x))``.  ``ffn`` (and then ``ffn_norm``) may be None:
     the layer is its mixer alone.  ``post_norm`` is
     ``x <- norm(residual_scale * x + mixer(x)); x <- norm(residual_scale * x + ffn(x))``: the
-    sublayers read the stream itself and the norms come after the sums."""
+    sublayers read the stream itself and the norms come after the sums.  ``sublayer_norm`` is
+    ``x += norm(mixer(x)); x += norm(ffn(x))``: the sublayers read the stream itself and a norm
+    is applied to a sublayer's output alone.  ``side`` (with ``side_norm``): one more sublayer
+    that runs last in the same way (only in ``sublayer_norm``)."""
     mixer: Any
     ffn: Any
-    mixer_norm: NormSpec
-    ffn_norm: Optional[NormSpec]
+    mixer_norm: Any
+    ffn_norm: Optional[Any]
     arrangement: str = "pre_norm"
     residual_scale: float = 1.0
+    side: Any = None
+    side_norm: Optional[Any] = None
 
 
 @dataclass(frozen=True)
@@ -234,7 +317,7 @@ class ModelSpec:
     hidden: int
     layers: Tuple[BlockSpec, ...]
     schedule: Tuple[ScheduleEntry, ...]
-    final_norm: NormSpec
+    final_norm: Any
     tie_lm_head: bool
     max_positions: int
     embed_scale: float = 1.0
@@ -244,6 +327,7 @@ class ModelSpec:
     embedding: Any = None
     head: Any = None
     pass_offsets: int = 0                   # rows of the table that schedule entries add to the stream
+    tables: Tuple[Any, ...] = ()            # matrices that parts of several layers read (``TableSpec``)
 
     def embedding_spec(self) -> Any:
         return self.embedding if self.embedding is not None else \

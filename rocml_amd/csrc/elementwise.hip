@@ -271,23 +271,23 @@ ROCML_EXPORT int rocml_swiglu(const void* gu, int in_dtype, void* out, int out_d
 // rocml-kernels/kernels/rope.hip:23-27).  inv_freq[i] = theta^(-2i/rot_dim) comes from the host.
 __global__ void rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq,
                                   float* __restrict__ cos_t, float* __restrict__ sin_t, int half,
-                                  long long total) {
+                                  long long total, float scale) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
     long long t = idx / half;
     int i = (int)(idx - t * half);
     double a = (double)pos[t] * inv_freq[i];
-    cos_t[idx] = (float)cos(a);
-    sin_t[idx] = (float)sin(a);
+    cos_t[idx] = (float)cos(a) * scale;       // scale: one factor on every cosine and sine (1: none)
+    sin_t[idx] = (float)sin(a) * scale;
 }
 
 ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float* cos_t, float* sin_t,
-                                  int n_tokens, int half, hipStream_t stream) {
+                                  int n_tokens, int half, float scale, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && half > 0, "rope_table: bad sizes T=%d half=%d", n_tokens, half);
     long long total = (long long)n_tokens * half;
     if (total == 0) return 0;
     rope_table_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(pos, inv_freq, cos_t, sin_t,
-                                                                           half, total);
+                                                                           half, total, scale);
     ROCML_CHECK_LAUNCH("rope_table");
     return 0;
 }
@@ -320,7 +320,9 @@ __global__ void qk_norm_rope_append_kernel(
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
     int rows_per_token, int pairing, int first_row, const float* __restrict__ bias, int dv,
-    float qt_coef, int qt_every) {
+    float qt_coef, int qt_every, const float* __restrict__ span_inv) {
+    // span_inv (may be null): [T, 2], the norm's factor of a token's whole q row and whole k row; the gains then
+    // have one number per column of the q (k) projection, and a head takes its own part of them.
     // qt_coef, qt_every: the queries' stretch with their position (after the norm); every = 0: none.
     // bias (may be null): one number per column of the packed row, added to the projection's sums.
     // dv: the size of a value head; the value rows start behind the Hq + Hkv rows of d numbers.
@@ -362,7 +364,13 @@ __global__ void qk_norm_rope_append_kernel(
     }
     const float* gain = kind == 0 ? q_gain : (kind == 1 ? k_gain : nullptr);
     if (gain) {
-        float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+        float inv;
+        if (span_inv) {
+            inv = span_inv[(size_t)t * 2 + kind];
+            gain += (size_t)(kind == 0 ? r : r - hq) * d;
+        } else {
+            inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+        }
 #pragma unroll
         for (int j = 0; j < QK_PER_LANE; ++j) {
             int e = lane + j * WAVE;
@@ -459,7 +467,7 @@ qk_norm_rope_rows_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     TO* __restrict__ q_out, TO* __restrict__ kcache, const int* __restrict__ block_table, int bt_width,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token,
-    int first_row, const float* __restrict__ bias, float qt_coef, int qt_every) {
+    int first_row, const float* __restrict__ bias, float qt_coef, int qt_every, const float* __restrict__ span_inv) {
     constexpr int HJ = QK_PER_LANE / 2;
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     long long total = (long long)n_tokens * rows_per_token;
@@ -491,10 +499,16 @@ qk_norm_rope_rows_kernel(
         bool is_q = rr[i] < hq;
         const float* gain = is_q ? q_gain : k_gain;
         if (gain) {
-            float ss = 0.f;
+            float inv;
+            if (span_inv) {          // the norm spans the token's whole q (k) row: its factor is given, the gain is the head's part
+                inv = span_inv[(size_t)tok[i] * 2 + (is_q ? 0 : 1)];
+                gain += (size_t)(is_q ? rr[i] : rr[i] - hq) * d;
+            } else {
+                float ss = 0.f;
 #pragma unroll
-            for (int j = 0; j < QK_PER_LANE; ++j) ss = fmaf(v[i][j], v[i][j], ss);
-            float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+                for (int j = 0; j < QK_PER_LANE; ++j) ss = fmaf(v[i][j], v[i][j], ss);
+                inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+            }
 #pragma unroll
             for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = v[i][j] * inv * gain[lane + j * WAVE];
         }
@@ -572,7 +586,10 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, int pairing, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
     const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
-    long long split_stride, const float* bias, int dv, float qt_coef, int qt_every, hipStream_t stream) {
+    long long split_stride, const float* bias, int dv, float qt_coef, int qt_every, const float* span_inv,
+    hipStream_t stream) {
+    // span_inv (may be null): [T, 2] factors of a norm over a token's whole q row and whole k row (qk_span_stats);
+    // q_gain and k_gain then have hq * d and hkv * d numbers.
     // bias (may be null): [ld] numbers added to the projection's sums; dv (0: d): value head size.
     // qt_coef, qt_every: a query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1)
     // after its norm (every = 0: not).
@@ -592,6 +609,8 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
                   "qk_norm_rope_append: cache arguments missing");
     ROCML_REQUIRE(q_out || write_kv, "qk_norm_rope_append: nothing to write");
+    ROCML_REQUIRE(!span_inv || (n_splits == 1 && q_gain && k_gain),
+                  "qk_norm_rope_append: a norm over the whole projection needs a complete projection and both gains");
     if (n_tokens == 0) return 0;
     // prompts: the values go through the transposing tile kernel, the row kernel does q and k
     bool v_tiled = write_kv && n_splits == 1 && n_tokens >= VT_TOKENS;
@@ -614,12 +633,12 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv, qt_coef, qt_every)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv, qt_coef, qt_every, span_inv)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
         rot ? sin_t : nullptr, (TO*)q_out, (TO*)kcache, block_table, bt_width, token_seq,       \
-        token_pos, page_size, rows_per_token, first_row, bias, qt_coef, qt_every)
+        token_pos, page_size, rows_per_token, first_row, bias, qt_coef, qt_every, span_inv)
 #define LAUNCH(TI, TO)                                                                          \
     {                                                                                           \
         if (many_rows) { if (per_lane == 2) LAUNCH_ROWS(TI, TO, 2); else LAUNCH_ROWS(TI, TO, 4); } \
@@ -642,6 +661,46 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
 #undef LAUNCH_N
 #undef LAUNCH_ROWS
     ROCML_CHECK_LAUNCH("qk_norm_rope_append");
+    return 0;
+}
+
+// ---- factors of a norm over a token's whole q row and whole k row ---------------------------
+// inv[t, 0] = 1 / sqrt(mean over the q_width leading columns of (row + bias)^2 + eps), inv[t, 1] the same over the
+// k_width columns behind them.  One block per token; 32-bit.
+template <typename TI>
+__global__ void __launch_bounds__(EW_BLOCK)
+qk_span_stats_kernel(const TI* __restrict__ qkv, int ld, int q_width, int k_width, const float* __restrict__ bias,
+                     float eps, float* __restrict__ inv) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    const TI* row = qkv + (size_t)blockIdx.x * ld;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < q_width; i += EW_BLOCK) {
+        float v = Elem<TI>::load(row + i) + (bias ? bias[i] : 0.f);
+        sq = fmaf(v, v, sq);
+    }
+    for (int i = threadIdx.x; i < k_width; i += EW_BLOCK) {
+        float v = Elem<TI>::load(row + q_width + i) + (bias ? bias[q_width + i] : 0.f);
+        sk = fmaf(v, v, sk);
+    }
+    sq = block_sum(sq, scratch);
+    sk = block_sum(sk, scratch);
+    if (threadIdx.x == 0) {
+        inv[(size_t)blockIdx.x * 2] = 1.0f / sqrtf(sq / (float)q_width + eps);
+        inv[(size_t)blockIdx.x * 2 + 1] = 1.0f / sqrtf(sk / (float)k_width + eps);
+    }
+}
+
+ROCML_EXPORT int rocml_qk_span_stats(const void* qkv, int dtype, int ld, int n_tokens, int q_width, int k_width,
+                                     const float* bias, float eps, float* inv, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && q_width > 0 && k_width > 0 && ld >= q_width + k_width && qkv && inv,
+                  "qk_span_stats: bad sizes T=%d q=%d k=%d ld=%d", n_tokens, q_width, k_width, ld);
+    if (n_tokens == 0) return 0;
+    if (dtype == ROCML_F32)
+        qk_span_stats_kernel<float><<<n_tokens, EW_BLOCK, 0, stream>>>((const float*)qkv, ld, q_width, k_width, bias, eps, inv);
+    else if (dtype == ROCML_BF16)
+        qk_span_stats_kernel<bf16_t><<<n_tokens, EW_BLOCK, 0, stream>>>((const bf16_t*)qkv, ld, q_width, k_width, bias, eps, inv);
+    else return rocml_fail("qk_span_stats: unknown dtype code %d", dtype);
+    ROCML_CHECK_LAUNCH("qk_span_stats");
     return 0;
 }
 
@@ -823,24 +882,26 @@ ROCML_EXPORT int rocml_rope_heads(const float* q, int ldq, int head_stride, int 
     return 0;
 }
 
-// y[t, i] = y[t, i] * sigmoid(g[t, i]) with g 32-bit in rows of ldg numbers: an output gate.
+// y[t, i] = y[t, i] * sigmoid(g[t, i / group]) with g 32-bit in rows of ldg numbers: an output gate,
+// one number per value (group = 1) or one per run of `group` values (a head).
 template <typename T>
-__global__ void sigmoid_gate_kernel(T* __restrict__ y, const float* __restrict__ g, int ldg, int n, long long total) {
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, const float* __restrict__ g, int ldg, int n, int group, long long total) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
     long long t = idx / n;
     int i = (int)(idx - t * n);
-    float gate = 1.0f / (1.0f + expf(-g[(size_t)t * ldg + i]));
+    float gate = 1.0f / (1.0f + expf(-g[(size_t)t * ldg + i / group]));
     Elem<T>::store(y + idx, Elem<T>::load(y + idx) * gate);
 }
 
-ROCML_EXPORT int rocml_sigmoid_gate(void* y, int dtype, const float* g, int ldg, int n_rows, int n, hipStream_t stream) {
-    ROCML_REQUIRE(n_rows >= 0 && n > 0 && ldg >= n, "sigmoid_gate: bad sizes rows=%d n=%d ld=%d", n_rows, n, ldg);
+ROCML_EXPORT int rocml_sigmoid_gate(void* y, int dtype, const float* g, int ldg, int n_rows, int n, int group, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0 && group > 0 && n % group == 0 && ldg >= n / group,
+                  "sigmoid_gate: bad sizes rows=%d n=%d group=%d ld=%d", n_rows, n, group, ldg);
     long long total = (long long)n_rows * n;
     if (total == 0) return 0;
     int grid = ceil_div(total, EW_BLOCK);
-    if (dtype == ROCML_F32) sigmoid_gate_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((float*)y, g, ldg, n, total);
-    else if (dtype == ROCML_BF16) sigmoid_gate_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((bf16_t*)y, g, ldg, n, total);
+    if (dtype == ROCML_F32) sigmoid_gate_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((float*)y, g, ldg, n, group, total);
+    else if (dtype == ROCML_BF16) sigmoid_gate_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((bf16_t*)y, g, ldg, n, group, total);
     else return rocml_fail("sigmoid_gate: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("sigmoid_gate");
     return 0;
@@ -1142,6 +1203,195 @@ ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float 
         sum_norm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, br, alpha, c, gain, eps, n, (bf16_t*)copy);
     else return rocml_fail("sum_norm: unknown dtype code %d", copy_dtype);
     ROCML_CHECK_LAUNCH("sum_norm");
+    return 0;
+}
+
+// ---- norm of a sublayer's output, added to the stream ------------------------------------------
+// x[t, :] += f(y[t, :]) in 32-bit, f a layer norm, (y - mean) / sqrt(var + eps) * gain + bias with var the mean
+// of the squared deviations from the mean (LAYER), or y / sqrt(mean(y^2) + eps) * gain; `copy` (may be null) gets
+// the new x in another type, for the products that read it next.  One block per row.
+template <typename TC, bool LAYER>
+__global__ void __launch_bounds__(EW_BLOCK)
+norm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
+                const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    size_t row = (size_t)blockIdx.x * n;
+    float mean = 0.f;
+    if (LAYER) {
+        float s = 0.f;
+        for (int i = threadIdx.x; i < n; i += EW_BLOCK) s += y[row + i];
+        mean = block_sum(s, scratch) / (float)n;
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float d = y[row + i] - mean;
+        ss = fmaf(d, d, ss);
+    }
+    float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float v = (y[row + i] - mean) * inv * gain[i];
+        if (LAYER && bias) v += bias[i];
+        v += x[row + i];
+        x[row + i] = v;
+        if (copy) Elem<TC>::store(copy + row + i, v);
+    }
+}
+
+// The same for rows of up to 8192 values that are a multiple of 4: the row stays in registers and all
+// loads are issued at once.
+template <typename TC, bool LAYER, int VEC>
+__global__ void __launch_bounds__(EW_BLOCK)
+norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
+                    const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    size_t row = (size_t)blockIdx.x * n;
+    int nv = n / 4;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 yv[VEC], xv[VEC], gv[VEC], bv[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        bool ok = i < nv;
+        yv[j] = ok ? ((const float4*)(y + row))[i] : zero4;
+        xv[j] = ok ? ((const float4*)(x + row))[i] : zero4;
+        gv[j] = ok ? ((const float4*)gain)[i] : zero4;
+        bv[j] = (ok && LAYER && bias) ? ((const float4*)bias)[i] : zero4;
+    }
+    float mean = 0.f;
+    if (LAYER) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) s += (yv[j].x + yv[j].y) + (yv[j].z + yv[j].w);
+        mean = block_sum(s, scratch) / (float)n;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        if (threadIdx.x + j * EW_BLOCK < nv) {
+            yv[j].x -= mean; yv[j].y -= mean; yv[j].z -= mean; yv[j].w -= mean;
+        }
+        ss = fmaf(yv[j].x, yv[j].x, ss); ss = fmaf(yv[j].y, yv[j].y, ss);
+        ss = fmaf(yv[j].z, yv[j].z, ss); ss = fmaf(yv[j].w, yv[j].w, ss);
+    }
+    float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        if (i >= nv) continue;
+        float4 v;
+        v.x = xv[j].x + (yv[j].x * inv * gv[j].x + bv[j].x);
+        v.y = xv[j].y + (yv[j].y * inv * gv[j].y + bv[j].y);
+        v.z = xv[j].z + (yv[j].z * inv * gv[j].z + bv[j].z);
+        v.w = xv[j].w + (yv[j].w * inv * gv[j].w + bv[j].w);
+        ((float4*)(x + row))[i] = v;
+        if (copy) store4(copy + row + 4 * (size_t)i, v.x, v.y, v.z, v.w);
+    }
+}
+
+template <typename TC, bool LAYER>
+static void launch_norm_add(float* x, const float* y, const float* gain, const float* bias, float eps, int n_rows, int n,
+                            TC* copy, hipStream_t stream) {
+    bool vec = n % 4 == 0 && n <= 4 * EW_BLOCK * RN_MAX_VEC && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
+               (uintptr_t)gain % 16 == 0 && (!bias || (uintptr_t)bias % 16 == 0) && (!copy || (uintptr_t)copy % 8 == 0);
+    int v = ceil_div(n / 4, EW_BLOCK);
+#define NAV(V_) norm_add_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy)
+    if (!vec) norm_add_kernel<TC, LAYER><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy);
+    else if (v <= 1) NAV(1);
+    else if (v <= 2) NAV(2);
+    else if (v <= 4) NAV(4);
+    else NAV(8);
+#undef NAV
+}
+
+ROCML_EXPORT int rocml_norm_add(float* x, const float* y, int n_rows, int n, const float* gain, const float* bias,
+                                float eps, int layer, void* copy, int copy_dtype, hipStream_t stream) {
+    // layer = 1: layer norm (mean taken off, bias added if given); 0: root-mean-square norm (bias is not read)
+    ROCML_REQUIRE(n_rows >= 0 && n > 0 && x && y && gain, "norm_add: bad arguments rows=%d n=%d", n_rows, n);
+    ROCML_REQUIRE(!copy || copy_dtype == ROCML_F32 || copy_dtype == ROCML_BF16, "norm_add: unknown dtype code %d", copy_dtype);
+    if (n_rows == 0) return 0;
+    bool half = copy && copy_dtype == ROCML_BF16;
+    if (layer) {
+        if (half) launch_norm_add<bf16_t, true>(x, y, gain, bias, eps, n_rows, n, (bf16_t*)copy, stream);
+        else launch_norm_add<float, true>(x, y, gain, bias, eps, n_rows, n, (float*)copy, stream);
+    } else {
+        if (half) launch_norm_add<bf16_t, false>(x, y, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, stream);
+        else launch_norm_add<float, false>(x, y, gain, nullptr, eps, n_rows, n, (float*)copy, stream);
+    }
+    ROCML_CHECK_LAUNCH("norm_add");
+    return 0;
+}
+
+// ---- layer norm ------------------------------------------------------------------------------
+// out[r, :] = (x[src(r), :] - mean) / sqrt(var + eps) * gain + bias, var the mean of the squared deviations from
+// the mean; `rows` optionally gathers source rows.  32-bit statistics, one block per row.
+template <typename TO>
+__global__ void __launch_bounds__(EW_BLOCK)
+layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ gain,
+                 const float* __restrict__ bias, float eps, int n, TO* __restrict__ out) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    const float* xin = x + (size_t)(rows ? rows[blockIdx.x] : blockIdx.x) * n;
+    TO* o = out + (size_t)blockIdx.x * n;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) s += xin[i];
+    float mean = block_sum(s, scratch) / (float)n;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float d = xin[i] - mean;
+        ss = fmaf(d, d, ss);
+    }
+    float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK)
+        Elem<TO>::store(o + i, (xin[i] - mean) * inv * gain[i] + (bias ? bias[i] : 0.f));
+}
+
+ROCML_EXPORT int rocml_layernorm(const float* x, const int* rows, int n_out, int n, const float* gain, const float* bias,
+                                 float eps, void* out, int out_dtype, hipStream_t stream) {
+    ROCML_REQUIRE(n_out >= 0 && n > 0 && x && gain && out, "layernorm: bad arguments rows=%d n=%d", n_out, n);
+    if (n_out == 0) return 0;
+    if (out_dtype == ROCML_F32) layernorm_kernel<float><<<n_out, EW_BLOCK, 0, stream>>>(x, rows, gain, bias, eps, n, (float*)out);
+    else if (out_dtype == ROCML_BF16) layernorm_kernel<bf16_t><<<n_out, EW_BLOCK, 0, stream>>>(x, rows, gain, bias, eps, n, (bf16_t*)out);
+    else return rocml_fail("layernorm: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("layernorm");
+    return 0;
+}
+
+// ---- an input that depends on the token's id, gated -----------------------------------------
+// out[t, j] = act(g[t, j]) * table[ids[t], col0 + j] for j < dim: g 32-bit [T, dim], the table [vocab, cols] in its own
+// type, act = gelu_tanh, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))) (act = 0), or the identity (act = 1).
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename TT, typename TO>
+__global__ void token_side_gate_kernel(const float* __restrict__ g, const TT* __restrict__ table, const int* __restrict__ ids,
+                                       int cols, int col0, int dim, int vocab, int act, TO* __restrict__ out, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / dim;
+    int j = (int)(idx - t * dim);
+    int id = ids[t];
+    float e = (id >= 0 && id < vocab) ? Elem<TT>::load(table + (size_t)id * cols + col0 + j) : 0.f;
+    float z = g[idx];
+    Elem<TO>::store(out + idx, (act == 0 ? gelu_tanh_f(z) : z) * e);
+}
+
+ROCML_EXPORT int rocml_token_side_gate(const float* g, const void* table, int table_dtype, const int* ids, int n_tokens,
+                                       int cols, int col0, int dim, int vocab, int act, void* out, int out_dtype,
+                                       hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && dim > 0 && col0 >= 0 && col0 + dim <= cols && vocab > 0 && g && table && ids && out,
+                  "token_side_gate: bad arguments T=%d dim=%d col0=%d cols=%d", n_tokens, dim, col0, cols);
+    ROCML_REQUIRE(act == 0 || act == 1, "token_side_gate: unknown activation %d", act);
+    long long total = (long long)n_tokens * dim;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+#define TSG(TT, TO) token_side_gate_kernel<TT, TO><<<grid, EW_BLOCK, 0, stream>>>(g, (const TT*)table, ids, cols, col0, dim, vocab, act, (TO*)out, total)
+    if (table_dtype == ROCML_F32 && out_dtype == ROCML_F32) TSG(float, float);
+    else if (table_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) TSG(bf16_t, bf16_t);
+    else if (table_dtype == ROCML_BF16 && out_dtype == ROCML_F32) TSG(bf16_t, float);
+    else if (table_dtype == ROCML_F32 && out_dtype == ROCML_BF16) TSG(float, bf16_t);
+    else return rocml_fail("token_side_gate: unknown dtype codes %d, %d", table_dtype, out_dtype);
+#undef TSG
+    ROCML_CHECK_LAUNCH("token_side_gate");
     return 0;
 }
 

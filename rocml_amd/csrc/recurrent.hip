@@ -538,6 +538,204 @@ ROCML_EXPORT int rocml_ssd_scan(const float* xbc, int ldx, const float* dtsrc, i
     return 0;
 }
 
+// ---- the matrix memory (mLSTM) --------------------------------------------------------
+// Per head and token t, with q_t (times q_scale), k_t [dk] and v_t [dv] from columns of the 32-bit projection and
+// the raw gates i~, f~ from two more of its columns:
+//     i = cap tanh((i~ + bi) / cap),   f = logsigmoid(cap tanh((f~ + bf) / cap)),
+//     m' = max(f + m, i),   a = exp(f + m - m'),   b = exp(i - m'),
+//     S <- a S + b k v^T,   n <- a n + b k,   o = S^T q / (max(|n . q|, exp(-m')) + floor).
+// The columns of S (one per value) do not depend on each other, and n is one more such column whose value is
+// always 1: a block takes one sequence, one head and SC_PT values, and walks the sequence's tokens in order, as
+// the recurrence above does.  Thread (pair of columns, r) keeps entries d = r * NI .. of its two columns and of n in
+// registers; the 16 threads of a pair add their parts of S^T q and n . q with cross-lane additions inside their
+// row of 16 lanes.  Every block of a head keeps n and m for itself (a block never reads what another writes in
+// the same launch).  State layouts: S [slot, H, dv, dk] (a column's dk entries side by side), n [slot, H, tiles, dk],
+// m [slot, H, tiles], tiles = ceil(dv / SC_PT); all zero when a sequence starts.  A step of one token per sequence
+// and a step of a prompt run the same arithmetic per token.
+constexpr int ML_TC = 32;
+
+__device__ __forceinline__ float rc_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <int NI>
+__global__ void __launch_bounds__(RC_BLOCK)
+mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0, int v_col0, int i_col0, int f_col0,
+                  const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale, float floor_,
+                  float* __restrict__ s_state, float* __restrict__ n_state, float* __restrict__ m_state,
+                  const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, float* __restrict__ out,
+                  int n_heads, int dk, int dv, int tiles) {
+    extern __shared__ float4 ml_smem4[];
+    constexpr int NP = SC_R * NI;              // padded length of a q or k row
+    float* ks = (float*)ml_smem4;              // [ML_TC][NP]
+    float* qs = ks + ML_TC * NP;               // [ML_TC][NP]
+    float* vs = qs + ML_TC * NP;               // [ML_TC][SC_PT]
+    float* os = vs + ML_TC * SC_PT;            // [ML_TC][SC_PT]
+    float* gs = os + ML_TC * SC_PT;            // [ML_TC][2]: log input gate, log forget gate
+    int tile = blockIdx.x, p0 = tile * SC_PT, head = blockIdx.y, b = blockIdx.z;
+    int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
+    int first = cu_seqlens[b], n_tok = cu_seqlens[b + 1] - first;
+    size_t slot_head = (size_t)seq_slots[b] * n_heads + head;
+    float* st_head = s_state + slot_head * dv * dk;
+    float* n_mine = n_state + (slot_head * tiles + tile) * dk;
+    float s[SC_PP][NI], nn[NI];
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        sc_load_state<NI>(s[j], st_head + (size_t)min(p, dv - 1) * dk, r, dk, p < dv);
+    }
+    sc_load_state<NI>(nn, n_mine, r, dk, true);
+    float m = m_state[slot_head * tiles + tile];
+    float bi = i_bias ? i_bias[head] : 0.f, bf = f_bias ? f_bias[head] : 0.f;
+    for (int c0 = 0; c0 < n_tok; c0 += ML_TC) {
+        int nt = min(ML_TC, n_tok - c0);
+        __syncthreads();                          // the previous chunk's outputs have been written out
+        for (int i = tid; i < nt * NP; i += RC_BLOCK) {
+            int tt = i / NP, d = i - tt * NP;
+            const float* row = proj + (size_t)(first + c0 + tt) * ld + (size_t)head * dk + d;
+            bool ok = d < dk;
+            ks[i] = ok ? row[k_col0] : 0.f;
+            qs[i] = ok ? row[q_col0] * q_scale : 0.f;
+        }
+        for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
+            int tt = i / SC_PT, pp = i - tt * SC_PT;
+            vs[i] = p0 + pp < dv ? proj[(size_t)(first + c0 + tt) * ld + v_col0 + (size_t)head * dv + p0 + pp] : 0.f;
+        }
+        if (tid < nt) {
+            const float* row = proj + (size_t)(first + c0 + tid) * ld;
+            gs[2 * tid] = cap * tanhf((row[i_col0 + head] + bi) / cap);
+            gs[2 * tid + 1] = rc_logsigmoid(cap * tanhf((row[f_col0 + head] + bf) / cap));
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            float2 g = *(const float2*)(gs + 2 * tt);
+            float2 xv = *(const float2*)(vs + tt * SC_PT + pl * SC_PP);
+            float kv[NI], qv[NI];
+            const float* kt = ks + tt * NP + r * NI;
+            const float* qt = qs + tt * NP + r * NI;
+            if (NI % 4 == 0) {
+#pragma unroll
+                for (int i = 0; i < NI; i += 4) {
+                    float4 k4 = *(const float4*)(kt + i), q4 = *(const float4*)(qt + i);
+                    kv[i] = k4.x; kv[i + 1] = k4.y; kv[i + 2] = k4.z; kv[i + 3] = k4.w;
+                    qv[i] = q4.x; qv[i + 1] = q4.y; qv[i + 2] = q4.z; qv[i + 3] = q4.w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NI; ++i) { kv[i] = kt[i]; qv[i] = qt[i]; }
+            }
+            float m_new = fmaxf(g.y + m, g.x);
+            float a = expf(g.y + m - m_new), bb = expf(g.x - m_new);
+            m = m_new;
+            float bv0 = bb * xv.x, bv1 = bb * xv.y, q0 = 0.f, q1 = 0.f, nq = 0.f;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                s[0][i] = fmaf(a, s[0][i], bv0 * kv[i]);
+                s[1][i] = fmaf(a, s[1][i], bv1 * kv[i]);
+                nn[i] = fmaf(a, nn[i], bb * kv[i]);
+                q0 = fmaf(s[0][i], qv[i], q0);
+                q1 = fmaf(s[1][i], qv[i], q1);
+                nq = fmaf(nn[i], qv[i], nq);
+            }
+            q0 = row16_sum(q0);
+            q1 = row16_sum(q1);
+            nq = row16_sum(nq);
+            float den = fmaxf(fabsf(nq), expf(-m)) + floor_;
+            if (r == 0) *(float2*)(os + tt * SC_PT + pl * SC_PP) = make_float2(q0 / den, q1 / den);
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
+            int tt = i / SC_PT, pp = i - tt * SC_PT;
+            if (p0 + pp < dv) out[(size_t)(first + c0 + tt) * n_heads * dv + (size_t)head * dv + p0 + pp] = os[i];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        sc_store_state<NI>(s[j], st_head + (size_t)min(p, dv - 1) * dk, r, dk, p < dv);
+    }
+    if (pl == 0) sc_store_state<NI>(nn, n_mine, r, dk, true);
+    if (tid == 0) m_state[slot_head * tiles + tile] = m;
+}
+
+ROCML_EXPORT int rocml_mlstm_tile() { return SC_PT; }
+
+ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_col0, int v_col0, int i_col0, int f_col0,
+                                  const float* i_bias, const float* f_bias, float cap, float q_scale, float floor_,
+                                  float* s_state, float* n_state, float* m_state, int n_slots, const int* cu_seqlens,
+                                  const int* seq_slots, int n_seqs, int n_tokens, float* out, int n_heads, int dk, int dv,
+                                  hipStream_t stream) {
+    ROCML_REQUIRE(n_heads > 0 && dk > 0 && dv > 0 && cap > 0.f, "mlstm_scan: bad sizes heads=%d dk=%d dv=%d cap=%g", n_heads,
+                  dk, dv, (double)cap);
+    ROCML_REQUIRE(dk <= 16 * SC_R, "mlstm_scan: a key size of %d exceeds %d", dk, 16 * SC_R);
+    ROCML_REQUIRE(q_col0 >= 0 && k_col0 >= 0 && v_col0 >= 0 && i_col0 >= 0 && f_col0 >= 0 && ld >= q_col0 + n_heads * dk &&
+                      ld >= k_col0 + n_heads * dk && ld >= v_col0 + n_heads * dv && ld >= i_col0 + n_heads && ld >= f_col0 + n_heads,
+                  "mlstm_scan: rows of %d are too short for their columns", ld);
+    ROCML_REQUIRE(proj && s_state && n_state && m_state && cu_seqlens && seq_slots && out && n_slots > 0,
+                  "mlstm_scan: missing arguments");
+    ROCML_REQUIRE(n_seqs >= 0 && n_seqs < 65536 && n_heads < 65536, "mlstm_scan: too many sequences or heads for one launch");
+    if (n_seqs == 0 || n_tokens == 0) return 0;
+    int tiles = ceil_div(dv, SC_PT);
+    dim3 grid(tiles, n_heads, n_seqs);
+    int ni = ceil_div(dk, SC_R);
+    ni = ni <= 4 ? ni : ni <= 6 ? 6 : ni <= 8 ? 8 : ni <= 12 ? 12 : 16;
+    size_t lds = (size_t)(2 * ML_TC * SC_R * ni + 2 * ML_TC * SC_PT + 2 * ML_TC) * sizeof(float);
+#define MSCAN(NI_)                                                                                                     \
+    mlstm_scan_kernel<NI_><<<grid, RC_BLOCK, lds, stream>>>(proj, ld, q_col0, k_col0, v_col0, i_col0, f_col0, i_bias, f_bias, \
+                                                            cap, q_scale, floor_, s_state, n_state, m_state, cu_seqlens,  \
+                                                            seq_slots, out, n_heads, dk, dv, tiles)
+    switch (ni) {
+        case 1: MSCAN(1); break;
+        case 2: MSCAN(2); break;
+        case 3: MSCAN(3); break;
+        case 4: MSCAN(4); break;
+        case 6: MSCAN(6); break;
+        case 8: MSCAN(8); break;
+        case 12: MSCAN(12); break;
+        default: MSCAN(16); break;
+    }
+#undef MSCAN
+    ROCML_CHECK_LAUNCH("mlstm_scan");
+    return 0;
+}
+
+// ---- norm of every head, gain, output gate ---------------------------------------------
+// out[t, h * dv + j] = o / sqrt(mean over the head's dv values of o^2 + eps) * gain[h * dv + j] * sigmoid(g[t, g_col0 + h * dv + j]):
+// o [T, H * dv] and g (rows of ldg numbers) 32-bit, the statistics 32-bit; a wave per (token, head).
+template <typename TO>
+__global__ void __launch_bounds__(RC_BLOCK)
+head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ g, int ldg, int g_col0,
+                      const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps) {
+    int lane = threadIdx.x & (WAVE - 1);
+    long long row = (long long)blockIdx.x * (RC_BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (row >= n_rows) return;
+    long long t = row / n_heads;
+    int h = (int)(row - t * n_heads);
+    const float* src = o + (size_t)row * dv;
+    float ss = 0.f;
+    for (int j = lane; j < dv; j += WAVE) ss = fmaf(src[j], src[j], ss);
+    float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+    const float* gr = g + (size_t)t * ldg + g_col0 + (size_t)h * dv;
+    for (int j = lane; j < dv; j += WAVE) {
+        float gate = 1.0f / (1.0f + expf(-gr[j]));
+        Elem<TO>::store(out + (size_t)row * dv + j, src[j] * inv * gain[(size_t)h * dv + j] * gate);
+    }
+}
+
+ROCML_EXPORT int rocml_head_norm_gate(const float* o, const float* g, int ldg, int g_col0, const float* gain, void* out,
+                                      int out_dtype, int n_tokens, int n_heads, int dv, float eps, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && dv > 0 && g_col0 >= 0 && ldg >= g_col0 + n_heads * dv && o && g && gain && out,
+                  "head_norm_gate: bad arguments T=%d heads=%d dv=%d ld=%d", n_tokens, n_heads, dv, ldg);
+    long long rows = (long long)n_tokens * n_heads;
+    if (rows == 0) return 0;
+    int grid = ceil_div(rows, RC_BLOCK / WAVE);
+    if (out_dtype == ROCML_F32)
+        head_norm_gate_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
+    else if (out_dtype == ROCML_BF16)
+        head_norm_gate_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
+    else return rocml_fail("head_norm_gate: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("head_norm_gate");
+    return 0;
+}
+
 // ---- gated norm in equal parts ------------------------------------------------------
 // out[t, i] = v / sqrt(mean over i's part of v^2 + eps) * gain[i],  v = y[t, i] * silu(z[t, i]):
 // the gate comes before the norm, and each of the `parts` equal parts of a row has a root mean

@@ -42,6 +42,7 @@ class StepContext:
     memo: Dict = field(default_factory=dict)
     block_tables: Dict = field(default_factory=dict)   # cache group name -> [B, width] int32
     want_rows: Optional[torch.Tensor] = None           # token rows whose logits are wanted
+    tables: Dict = field(default_factory=dict)         # the model's matrices that parts of several layers read, by name
 
     @property
     def is_decode(self) -> bool:

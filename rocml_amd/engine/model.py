@@ -42,6 +42,8 @@ class DecoderModel:
         self.head = build_head(spec.head_spec(), ctx)
         # rows that schedule entries add to the residual stream before they run (32-bit)
         self.pass_offset: Optional[torch.Tensor] = None
+        # matrices that parts of several layers read (each its own columns), by name; a step carries them
+        self.tables: Dict[str, torch.Tensor] = {}
         self.bound = False
         # whether a decode step may be recorded as a graph: every part must say so
         self.graph_safe = all(getattr(part, "graph_safe", True)
@@ -79,6 +81,8 @@ class DecoderModel:
                 specs[f"layers.{i}.{name}"] = p
         if self.spec.pass_offsets:
             specs["pass_offset.weight"] = ParamSpec((self.spec.pass_offsets, self.spec.hidden), role="gain", init="normal")
+        for t in self.spec.tables:
+            specs[f"tables.{t.name}"] = ParamSpec((t.rows, t.cols))
         specs.update(self.head.param_specs())
         return specs
 
@@ -93,6 +97,7 @@ class DecoderModel:
         self.head.bind({k: tensors[k] for k in self.head.param_specs()}, shared=self.embedding.shared_matrix())
         if self.spec.pass_offsets:
             self.pass_offset = tensors["pass_offset.weight"]
+        self.tables = {t.name: tensors[f"tables.{t.name}"] for t in self.spec.tables}
         self.bound = True
 
     def weight_bytes(self) -> int:
@@ -174,6 +179,7 @@ class DecoderModel:
         s = self.spec
         ws = step.workspace
         ws.drop_pending()
+        step.tables = self.tables
         x = ws.get("model.x", (step.n_tokens, s.hidden), torch.float32)
         self.embedding.forward(step, x)
         for i, entry in enumerate(s.schedule):

@@ -30,9 +30,13 @@ _SIGNATURES = {
         "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P, _P, _I, _P],
         "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P, _I, _LL, _P],
         "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _P],
-        "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
+        "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _F, _P],
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
-                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P],
+                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _P],
+        "rocml_qk_span_stats": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P],
+        "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P],
+        "rocml_layernorm": [_P, _P, _I, _I, _P, _P, _F, _P, _I, _P],
+        "rocml_token_side_gate": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
         "rocml_add_row_vector": [_P, _P, _I, _I, _P],
         "rocml_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _P],
@@ -40,7 +44,7 @@ _SIGNATURES = {
         "rocml_latent_window_plan": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P, _I, _P],
         "rocml_latent_window_gather": [_P, _I, _I, _I, _P, _I, _P, _P],
         "rocml_gate_heads": [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _P],
-        "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _P],
+        "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _I, _P],
         "rocml_sum_norm": [_P, _I, _I, _F, _F, _I, _P, _P, _P, _F, _P, _I, _P],
         "rocml_convert": [_P, _P, _I, _LL, _P],
     },
@@ -48,6 +52,9 @@ _SIGNATURES = {
         "rocml_causal_conv": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _P],
         "rocml_ssd_scan": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _I, _P],
         "rocml_gated_part_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+        "rocml_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _F, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
+        "rocml_mlstm_tile": [],
+        "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
     },
     "moe": {
         "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
@@ -244,7 +251,9 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False, 
         GATE_ACTIVATIONS[activation], 0.0 if limit is None else float(limit), float(up_offset), _stream()))
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+               scale: float = 1.0) -> None:
+    """``cos[t, i] = scale * cos(positions[t] * inv_freq[i])`` and the sines likewise (angles in 64-bit)."""
     _dev(positions, inv_freq, cos, sin)
     _want(positions, torch.int32, "positions")
     _want(inv_freq, torch.float64, "inverse frequencies")
@@ -254,7 +263,7 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tenso
     if cos.shape != (n, half) or sin.shape != (n, half):
         raise KernelError(f"rotation tables must be {(n, half)}")
     _check("elementwise", library("elementwise").rocml_rope_table(
-        _ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), n, half, _stream()))
+        _ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), n, half, float(scale), _stream()))
 
 
 ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}
@@ -267,7 +276,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
                         n_splits: int = 1, pairing: str = "halves", bias: Optional[torch.Tensor] = None,
-                        v_head_dim: Optional[int] = None, q_temp=None) -> None:
+                        v_head_dim: Optional[int] = None, q_temp=None, span_inv: Optional[torch.Tensor] = None) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
@@ -277,14 +286,16 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     one number per column of ``qkv``, added to the projection's sums.  ``v_head_dim``: the size of a
     value head when it is not ``head_dim`` (the value columns then follow the ``Hq + Hkv`` heads of
     ``head_dim``).  ``q_temp``: ``(coef, every)``; the query at position ``p`` is multiplied by
-    ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm."""
+    ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm.  ``span_inv``: ``[T, 2]`` 32-bit, the
+    factors of a norm over a token's whole q row and whole k row (``qk_span_stats``); the gains then
+    have one number per column of the q and of the k projection."""
     qt_coef, qt_every = (0.0, 0) if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
     if q_temp is not None and qt_every <= 0:
         raise KernelError(f"the period of the query's stretch must be positive, got {qt_every}")
     dv = head_dim if v_head_dim is None else int(v_head_dim)
     if pairing not in ROPE_PAIRINGS:
         raise KernelError(f"unknown rotation pairing {pairing!r}; known: {sorted(ROPE_PAIRINGS)}")
-    _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos, bias)
+    _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos, bias, span_inv)
     split_stride = 0
     if n_splits > 1:                      # [splits, T, ld] split-K partial sums, added in the kernel
         if qkv.dim() != 3 or qkv.shape[0] != n_splits:
@@ -296,11 +307,15 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         _want(bias, torch.float32, "projection bias")
         if bias.numel() != ld:
             raise KernelError(f"the bias has {bias.numel()} values for rows of {ld}")
-    for g in (q_gain, k_gain):
+    if span_inv is not None:
+        _want(span_inv, torch.float32, "norm factors")
+        if span_inv.shape != (n_tokens, 2) or n_splits > 1 or q_gain is None or k_gain is None:
+            raise KernelError("a norm over the whole projection needs [tokens, 2] factors, a complete projection and both gains")
+    for g, heads in ((q_gain, n_heads), (k_gain, n_kv_heads)):
         if g is not None:
             _want(g, torch.float32, "head norm gain")
-            if g.numel() != head_dim:
-                raise KernelError(f"head norm gain has {g.numel()} values for head size {head_dim}")
+            if g.numel() != (head_dim if span_inv is None else heads * head_dim):
+                raise KernelError(f"norm gain has {g.numel()} values for {heads} heads of size {head_dim}")
     if cos is not None:
         if cos.shape != (n_tokens, rot_dim // 2) or sin is None or sin.shape != cos.shape:
             raise KernelError(f"rotation tables must be {(n_tokens, rot_dim // 2)}")
@@ -325,7 +340,76 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out if q_out is not None else k_cache), _ptr(block_table), bt_width, _ptr(token_seq),
         _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _ptr(bias), dv, qt_coef, qt_every,
-        _stream()))
+        _ptr(span_inv), _stream()))
+
+
+def qk_span_stats(qkv: torch.Tensor, q_width: int, k_width: int, bias: Optional[torch.Tensor], eps: float,
+                  out: torch.Tensor) -> None:
+    """``out[t, 0] = 1 / sqrt(mean((qkv[t, :q_width] + bias)^2) + eps)`` and ``out[t, 1]`` the same over the
+    ``k_width`` columns behind them: the factors of a norm over a token's whole q row and whole k row."""
+    _dev(qkv, bias, out)
+    _want(out, torch.float32, "norm factors")
+    if qkv.dim() != 2 or out.shape != (qkv.shape[0], 2) or qkv.shape[1] < q_width + k_width:
+        raise KernelError("qk_span_stats: shapes do not fit")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() < q_width + k_width):
+        raise KernelError("qk_span_stats: the bias must be 32-bit and cover the q and k columns")
+    _check("elementwise", library("elementwise").rocml_qk_span_stats(
+        _ptr(qkv), _code(qkv), qkv.shape[1], qkv.shape[0], q_width, k_width, _ptr(bias), float(eps), _ptr(out), _stream()))
+
+
+def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+             layer: bool, copy: Optional[torch.Tensor] = None) -> None:
+    """``x += f(y)`` row by row in 32-bit: ``f`` a layer norm ``(y - mean) / sqrt(var + eps) * gain + bias``
+    (``layer``) or ``y / sqrt(mean(y^2) + eps) * gain``.  ``copy`` gets the new ``x`` in its own type."""
+    _dev(x, y, gain, bias, copy)
+    for t, what in ((x, "residual stream"), (y, "sublayer output"), (gain, "norm gain")):
+        _want(t, torch.float32, what)
+    if x.dim() != 2 or y.shape != x.shape or gain.numel() != x.shape[1] or (copy is not None and copy.shape != x.shape) \
+            or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != x.shape[1])):
+        raise KernelError("norm_add: shapes do not fit")
+    _check("elementwise", library("elementwise").rocml_norm_add(
+        _ptr(x), _ptr(y), x.shape[0], x.shape[1], _ptr(gain), _ptr(bias), float(eps), 1 if layer else 0, _ptr(copy),
+        _code(copy) if copy is not None else 0, _stream()))
+
+
+def layernorm(x: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float, out: torch.Tensor,
+              rows: Optional[torch.Tensor] = None) -> None:
+    """``out[r] = (x[s] - mean) / sqrt(var + eps) * gain + bias`` with ``s = rows[r]`` (or ``r``), ``var`` the
+    mean of the squared deviations; 32-bit ``x``, statistics 32-bit."""
+    _dev(x, gain, bias, out, rows)
+    _want(x, torch.float32, "norm input")
+    _want(gain, torch.float32, "norm gain")
+    n = x.shape[1]
+    n_out = out.shape[0]
+    if rows is not None:
+        _want(rows, torch.int32, "row indices")
+        if rows.numel() < n_out:
+            raise KernelError("layernorm: fewer row indices than output rows")
+    elif n_out != x.shape[0]:
+        raise KernelError("layernorm: output rows differ from input rows")
+    if out.shape[1] != n or gain.numel() != n or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != n)):
+        raise KernelError("layernorm: widths differ")
+    _check("elementwise", library("elementwise").rocml_layernorm(
+        _ptr(x), _ptr(rows), n_out, n, _ptr(gain), _ptr(bias), float(eps), _ptr(out), _code(out), _stream()))
+
+
+SIDE_ACTIVATIONS = {"gelu_tanh": 0, "identity": 1}
+
+
+def token_side_gate(g: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int, out: torch.Tensor,
+                    activation: str = "gelu_tanh") -> None:
+    """``out[t, j] = act(g[t, j]) * table[ids[t], col0 + j]`` for the 32-bit ``g [T, dim]``."""
+    _dev(g, table, ids, out)
+    _want(g, torch.float32, "gate")
+    _want(ids, torch.int32, "token ids")
+    if activation not in SIDE_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(SIDE_ACTIVATIONS)}")
+    n, dim = g.shape
+    if out.shape != g.shape or ids.numel() != n or table.dim() != 2 or col0 < 0 or col0 + dim > table.shape[1]:
+        raise KernelError("token_side_gate: shapes do not fit")
+    _check("elementwise", library("elementwise").rocml_token_side_gate(
+        _ptr(g), _ptr(table), _code(table), _ptr(ids), n, table.shape[1], col0, dim, table.shape[0],
+        SIDE_ACTIVATIONS[activation], _ptr(out), _code(out), _stream()))
 
 
 def add_row_vector(x: torch.Tensor, b: torch.Tensor) -> None:
@@ -442,18 +526,19 @@ def gate_heads(x: torch.Tensor, x_stride: int, gate: Optional[torch.Tensor], out
         _ptr(x), _code(x), x.shape[1], x_stride, _ptr(gate), ldg, _ptr(out), x.shape[0], n_heads, n, _stream()))
 
 
-def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:
-    """``y *= sigmoid(gate)`` for ``y [T, n]`` and the 32-bit ``gate [T, n]``, whose rows may be a
-    column range of a wider matrix."""
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor, group: int = 1) -> None:
+    """``y *= sigmoid(gate)`` for ``y [T, n]`` and the 32-bit ``gate [T, n / group]``, whose rows may be a
+    column range of a wider matrix; a gate value covers ``group`` neighbouring values of ``y`` (a head)."""
     _dev(y)
     if not gate.is_cuda:
         raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
     _want(gate, torch.float32, "gate")
-    if y.dim() != 2 or gate.shape != y.shape or gate.stride(1) != 1:
-        raise KernelError(f"gate {tuple(gate.shape)} does not fit {tuple(y.shape)}")
-    ldg = gate.stride(0) if y.shape[0] > 1 else max(gate.stride(0), y.shape[1])
+    if y.dim() != 2 or group <= 0 or y.shape[1] % group != 0 or gate.shape != (y.shape[0], y.shape[1] // group) \
+            or gate.stride(1) != 1:
+        raise KernelError(f"gate {tuple(gate.shape)} does not fit {tuple(y.shape)} in groups of {group}")
+    ldg = gate.stride(0) if y.shape[0] > 1 else max(gate.stride(0), gate.shape[1])
     _check("elementwise", library("elementwise").rocml_sigmoid_gate(_ptr(y), _code(y), _ptr(gate), ldg, y.shape[0],
-                                                                   y.shape[1], _stream()))
+                                                                   y.shape[1], group, _stream()))
 
 
 def sum_norm(x: torch.Tensor, branches: Sequence[torch.Tensor], branch_gains: Sequence[Optional[torch.Tensor]],
@@ -854,11 +939,15 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
     if v_cache.dtype != k_cache.dtype or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
             or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
         raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
-    for g in (q_gain, k_gain):
+    if span_inv is not None:
+        _want(span_inv, torch.float32, "norm factors")
+        if span_inv.shape != (n_tokens, 2) or n_splits > 1 or q_gain is None or k_gain is None:
+            raise KernelError("a norm over the whole projection needs [tokens, 2] factors, a complete projection and both gains")
+    for g, heads in ((q_gain, n_heads), (k_gain, n_kv_heads)):
         if g is not None:
             _want(g, torch.float32, "head norm gain")
-            if g.numel() != head_dim:
-                raise KernelError(f"head norm gain has {g.numel()} values for head size {head_dim}")
+            if g.numel() != (head_dim if span_inv is None else heads * head_dim):
+                raise KernelError(f"norm gain has {g.numel()} values for {heads} heads of size {head_dim}")
     if cos is not None:
         _want(cos, torch.float32, "rotation table")
         if cos.shape != (n_tokens, head_dim // 2) or sin is None or sin.shape != cos.shape or sin.dtype != cos.dtype:
@@ -994,6 +1083,63 @@ def gated_part_norm(y: torch.Tensor, z: torch.Tensor, z_col0: int, gain: torch.T
         raise KernelError("gated_part_norm: sizes differ")
     _check("recurrent", library("recurrent").rocml_gated_part_norm(
         _ptr(y), _ptr(z), z.shape[1], z_col0, _ptr(gain), _ptr(out), _code(out), rows, n, parts, float(eps), _stream()))
+
+
+MLSTM_COLUMNS = 32      # values of a head that one block of the matrix memory's kernel owns
+
+
+def mlstm_tiles(v_head_dim: int) -> int:
+    """Blocks per head of the matrix memory's kernel; each keeps the head's ``n`` and ``m`` for itself."""
+    return (v_head_dim + MLSTM_COLUMNS - 1) // MLSTM_COLUMNS
+
+
+def mlstm_scan(proj: torch.Tensor, q_col0: int, k_col0: int, v_col0: int, i_col0: int, f_col0: int,
+               i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], cap: float, q_scale: float, floor: float,
+               s_state: torch.Tensor, n_state: torch.Tensor, m_state: torch.Tensor, cu_seqlens: torch.Tensor,
+               seq_slots: torch.Tensor, out: torch.Tensor, n_heads: int, head_dim: int, v_head_dim: int) -> None:
+    """The matrix memory over the step's tokens, per sequence in order: with ``q`` (times ``q_scale``), ``k``,
+    ``v`` and the raw gates taken from columns of the 32-bit ``proj [T, ld]``,
+    ``i = cap tanh((raw_i + i_bias) / cap)``, ``f = logsigmoid(cap tanh((raw_f + f_bias) / cap))``,
+    ``m' = max(f + m, i)``, ``S <- exp(f + m - m') S + exp(i - m') k v^T``, ``n`` likewise with ``k`` alone,
+    ``out = S^T q / (max(|n . q|, exp(-m')) + floor)``.  States per slot: ``s_state [slots, H, dv, dk]``,
+    ``n_state [slots, H, tiles, dk]``, ``m_state [slots, H, tiles]`` with ``tiles = mlstm_tiles(dv)``; all 32-bit."""
+    _dev(proj, i_bias, f_bias, s_state, n_state, m_state, cu_seqlens, seq_slots, out)
+    for t, what in ((proj, "projection"), (s_state, "matrix state"), (n_state, "vector state"), (m_state, "maximum state"),
+                    (out, "memory output")):
+        _want(t, torch.float32, what)
+    lib = library("recurrent")
+    if lib.rocml_mlstm_tile() != MLSTM_COLUMNS:
+        raise KernelError("the matrix memory's kernel and its launcher disagree about a block's columns")
+    n_tokens, n_seqs, tiles = proj.shape[0], seq_slots.numel(), mlstm_tiles(v_head_dim)
+    slots = s_state.shape[0]
+    if s_state.shape != (slots, n_heads, v_head_dim, head_dim) or n_state.shape != (slots, n_heads, tiles, head_dim) \
+            or m_state.shape != (slots, n_heads, tiles):
+        raise KernelError(f"matrix memory states {tuple(s_state.shape)}, {tuple(n_state.shape)}, {tuple(m_state.shape)} "
+                          f"do not fit {n_heads} heads of {head_dim} x {v_head_dim}")
+    if out.shape != (n_tokens, n_heads * v_head_dim) or cu_seqlens.numel() != n_seqs + 1:
+        raise KernelError("matrix memory output or tables do not fit the step")
+    for b in (i_bias, f_bias):
+        if b is not None and (b.dtype != torch.float32 or b.numel() != n_heads):
+            raise KernelError("gate biases must be 32-bit with one number per head")
+    _check("recurrent", lib.rocml_mlstm_scan(
+        _ptr(proj), proj.shape[1], q_col0, k_col0, v_col0, i_col0, f_col0, _ptr(i_bias), _ptr(f_bias), float(cap),
+        float(q_scale), float(floor), _ptr(s_state), _ptr(n_state), _ptr(m_state), slots, _ptr(cu_seqlens), _ptr(seq_slots),
+        n_seqs, n_tokens, _ptr(out), n_heads, head_dim, v_head_dim, _stream()))
+
+
+def head_norm_gate(o: torch.Tensor, g: torch.Tensor, g_col0: int, gain: torch.Tensor, out: torch.Tensor, n_heads: int,
+                   eps: float) -> None:
+    """``out = rms_heads(o) * gain * sigmoid(g)``: every one of the ``n_heads`` equal parts of a row of the 32-bit
+    ``o [T, n]`` divided by its own root mean square; ``g`` is columns ``g_col0 ..`` of a 32-bit matrix."""
+    _dev(o, g, gain, out)
+    for t, what in ((o, "norm input"), (g, "gate"), (gain, "norm gain")):
+        _want(t, torch.float32, what)
+    rows, n = o.shape
+    if n % n_heads != 0 or gain.numel() != n or out.shape != o.shape or g.shape[0] != rows or g.shape[1] < g_col0 + n:
+        raise KernelError("head_norm_gate: sizes differ")
+    _check("recurrent", library("recurrent").rocml_head_norm_gate(
+        _ptr(o), _ptr(g), g.shape[1], g_col0, _ptr(gain), _ptr(out), _code(out), rows, n_heads, n // n_heads, float(eps),
+        _stream()))
 
 
 # ---- experts -----------------------------------------------------------------------------

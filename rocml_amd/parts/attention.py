@@ -35,8 +35,13 @@ class Attention(Mixer):
     def __init__(self, spec: AttentionSpec, ctx: BuildContext):
         if spec.n_heads % spec.n_kv_heads != 0:
             raise ConfigError(f"{spec.n_heads} query heads are not a multiple of {spec.n_kv_heads} key/value heads")
-        if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
-            raise ConfigError("the per-head norm must span the head size")
+        self.span = getattr(spec, "qk_norm_span", "head")
+        if self.span not in ("head", "projection"):
+            raise ConfigError(f"the norm of q and k spans a 'head' or the whole 'projection', got {self.span!r}")
+        if spec.qk_norm is not None and spec.qk_norm.size != (spec.head_dim if self.span == "head" else spec.n_heads * spec.head_dim):
+            raise ConfigError("the norm of q and k must span the head size, or with span 'projection' all query heads")
+        if self.span == "projection" and (spec.qk_norm is None or not getattr(spec.qk_norm, "learned", True)):
+            raise ConfigError("a norm over the whole projection needs learned gains")
         if spec.qk_norm is not None and spec.qk_norm.kind != "rmsnorm":
             # the norm of q and k runs inside the rotation and attention kernels, which know one kind
             raise ConfigError(f"the per-head norm must be of kind 'rmsnorm', got {spec.qk_norm.kind!r}")
@@ -54,7 +59,12 @@ class Attention(Mixer):
             raise ConfigError(f"the period of the query's stretch must be positive, got {spec.q_temp[1]}")
         # what only the norm-and-rotation kernel knows (the kernels that prepare their queries
         # themselves do not): a stretch of the query with its position, an output gate
-        self.separate_q = spec.q_temp is not None or spec.gate
+        # (and a norm over a token's whole q and k rows, whose factors a kernel of their own forms first)
+        self.separate_q = spec.q_temp is not None or spec.gate or self.span == "projection"
+        self.gate_per_head = bool(getattr(spec, "gate_per_head", False))
+        if self.gate_per_head and not spec.gate:
+            raise ConfigError("a gate per head needs the output gate switched on")
+        self.o_bias = spec.bias if getattr(spec, "o_bias", None) is None else bool(spec.o_bias)
         self.norm_learned = spec.qk_norm is None or getattr(spec.qk_norm, "learned", True)
         self.slopes: Optional[torch.Tensor] = None
         if spec.distance_slopes is not None and torch.device(ctx.device).type != "meta":
@@ -66,7 +76,7 @@ class Attention(Mixer):
         self.kv_dim = spec.n_kv_heads * spec.head_dim
         self.v_dim = spec.n_kv_heads * self.v_head_dim
         self.o_dim = spec.n_heads * self.v_head_dim
-        self.g_dim = self.o_dim if spec.gate else 0
+        self.g_dim = 0 if not spec.gate else (spec.n_heads if self.gate_per_head else self.o_dim)
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
         self.pairing = getattr(self.position, "pairing", "halves")
         if self.pairing not in ops.ROPE_PAIRINGS:
@@ -91,11 +101,13 @@ class Attention(Mixer):
         if s.bias:       # added in 32-bit to the products' sums
             specs.update({"q_proj.bias": ParamSpec((self.q_dim,), role="gain", init="normal"),
                           "k_proj.bias": ParamSpec((self.kv_dim,), role="gain", init="normal"),
-                          "v_proj.bias": ParamSpec((self.v_dim,), role="gain", init="normal"),
-                          "o_proj.bias": ParamSpec((s.hidden,), role="gain", init="normal")})
+                          "v_proj.bias": ParamSpec((self.v_dim,), role="gain", init="normal")})
+        if self.o_bias:
+            specs["o_proj.bias"] = ParamSpec((s.hidden,), role="gain", init="normal")
         if s.qk_norm is not None and self.norm_learned:
-            specs["q_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
-            specs["k_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
+            whole = self.span == "projection"       # one gain per column of the projection instead of one per head value
+            specs["q_norm.weight"] = ParamSpec((self.q_dim if whole else s.head_dim,), role="gain", init="gain")
+            specs["k_norm.weight"] = ParamSpec((self.kv_dim if whole else s.head_dim,), role="gain", init="gain")
         if s.gate:
             specs["g_proj.weight"] = ParamSpec((self.g_dim, s.hidden))
         return specs
@@ -108,7 +120,11 @@ class Attention(Mixer):
                                + ([tensors["g_proj.weight"]] if self.spec.gate else []), dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
         if self.spec.bias:
-            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
+            # (an output gate's columns, which come last in the product, have no bias: zeros stand for it)
+            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]
+                                   + ([torch.zeros(self.g_dim, dtype=torch.float32, device=self.w_o.device)] if self.g_dim else [])
+                                   ).contiguous()
+        if self.o_bias:
             self.b_o = tensors["o_proj.bias"]
         if self.spec.qk_norm is not None:
             if self.norm_learned:
@@ -195,7 +211,7 @@ class Attention(Mixer):
             # (the decode kernel that reads the projection adds four partial sums in one trip to memory
             # and further ones one after the other: K is cut into few pieces for it)
             # (the gate's columns are read where they lie: the product is then completed)
-            splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate,
+            splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate and self.span == "head",
                               max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
         if splits:      # the product's split-K partial sums; the next kernel adds them
             qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
@@ -234,17 +250,23 @@ class Attention(Mixer):
             else:
                 q = ws.get("attn.q", (n, self.q_dim), self.dtype)
                 bias = None if self.b_qkv is None else self.b_qkv[:rows]
+                span_inv = None
+                if self.span == "projection":
+                    if not owns_cache:
+                        raise ConfigError("a norm over the whole projection needs the layer's own keys")
+                    span_inv = ws.get("attn.span", (n, 2), torch.float32)
+                    ops.qk_span_stats(qkv, self.q_dim, self.kv_dim, bias, eps, span_inv)
                 ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                         cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
                                         step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing,
-                                        bias=bias, v_head_dim=self.v_head_dim, q_temp=s.q_temp)
+                                        bias=bias, v_head_dim=self.v_head_dim, q_temp=s.q_temp, span_inv=span_inv)
                 ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                               s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                               cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                               max_len=step.max_len, n_splits=self._decode_splits(step, cache),
                               v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink)
         if s.gate:
-            ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:rows])
+            ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:rows], group=self.v_head_dim if self.gate_per_head else 1)
         if self.b_o is not None:
             ws.flush_pending()
             ops.add_row_vector(x_accum, self.b_o)

@@ -5,7 +5,10 @@
 32-bit and the normalised copy has the activation type.
 
 ``post_norm`` norms after the sum: ``x <- norm(a x + mixer(x))``, then ``x <- norm(a x + ffn(x))`` with
-``a`` the block's ``residual_scale``; the sublayers read the stream itself."""
+``a`` the block's ``residual_scale``; the sublayers read the stream itself.
+
+``sublayer_norm`` norms a sublayer's output alone: ``x += norm(mixer(x))``, ``x += norm(ffn(x))`` and, if the
+layer has one, ``x += norm(side(x))``; the sublayers read the stream itself."""
 from __future__ import annotations
 
 from typing import Dict
@@ -208,3 +211,84 @@ class PostNormBlock(Part):
 
 
 register_block("post_norm", PostNormBlock)
+
+
+class SublayerNormBlock(Part):
+    """``x += norm1(mixer(x))``, ``x += norm2(ffn(x))``, ``x += norm3(side(x))`` (the last two may be absent).  A
+    sublayer reads the stream itself (in the compute type: a copy that the kernel before it wrote, the stream
+    itself in 32-bit) and writes its result to a buffer of the block; one kernel then norms that buffer, adds it
+    to the 32-bit stream and writes the copy for the next sublayer.  The norms are layer norms (weight and bias)
+    or root-mean-square norms (weight), each sublayer its own."""
+    takes_pending = False
+    takes_next_norm = False
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        self.dtype = ctx.dtype
+        self.hidden = spec.mixer_norm.size
+        self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
+                         "mixer": build_mixer(spec.mixer, ctx)}
+        if spec.ffn is not None:
+            self.children["ffn_norm"] = build_norm(spec.ffn_norm, ctx)
+            self.children["ffn"] = build_feed_forward(spec.ffn, ctx)
+        if spec.side is not None:
+            self.children["side_norm"] = build_norm(spec.side_norm, ctx)
+            self.children["side"] = build_feed_forward(spec.side, ctx)
+        self.mixer = self.children["mixer"]
+        self.ffn = self.children.get("ffn")
+        self.side = self.children.get("side")
+        for name in ("mixer_norm", "ffn_norm", "side_norm"):
+            norm = self.children.get(name)
+            if norm is not None and (not hasattr(norm, "gain") or not hasattr(norm, "eps")):
+                raise ConfigError("a block that norms its sublayers' outputs needs norms with a gain and an eps")
+        self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
+        self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
+        self.kernel_families = tuple(f for c in self.children.values() for f in getattr(c, "kernel_families", ()))
+
+    param_specs = PreNormBlock.param_specs
+    bind = PreNormBlock.bind
+    cache_request = PreNormBlock.cache_request
+
+    def flops(self, new_counts, starts) -> int:
+        return sum(part.flops(new_counts, starts) for part in (self.mixer, self.ffn, self.side) if part is not None)
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * self.hidden * (size + 4) + sum(part.activation_bytes(n_tokens)
+                                                         for part in (self.mixer, self.ffn, self.side) if part is not None)
+
+    _operand = PostNormBlock._operand
+
+    def _norm_add(self, step, x, y, norm) -> None:
+        copy = None
+        if self.dtype != torch.float32:
+            copy = step.workspace.get("block.stream_copy", tuple(x.shape), self.dtype)
+        ops.norm_add(x, y, norm.gain, getattr(norm, "bias", None), norm.eps, layer=bool(getattr(norm, "centred", False)), copy=copy)
+        if copy is not None:
+            step.memo[_COPY_KEY] = (x.data_ptr(), copy)
+
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+        ws = step.workspace
+        rs = stream(step)
+        ws.flush_pending()
+        rs.row_scale = rs.next_norm = None
+        try:
+            xb = self._operand(step, x)
+            y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
+            rs.overwrite = True
+            self.mixer.forward(step, xb, y, cache, owns_cache)
+            ws.flush_pending()
+            self._norm_add(step, x, y, self.children["mixer_norm"])
+            for part, norm in ((self.ffn, "ffn_norm"), (self.side, "side_norm")):
+                if part is None:
+                    continue
+                xb = self._operand(step, x)
+                y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
+                rs.overwrite = True
+                part.forward(step, xb, y)
+                ws.flush_pending()
+                self._norm_add(step, x, y, self.children[norm])
+        finally:
+            rs.overwrite = False
+
+
+register_block("sublayer_norm", SublayerNormBlock)

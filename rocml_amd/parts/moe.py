@@ -38,13 +38,22 @@ class RoutedExperts(FeedForward):
             if count <= 0 or spec.n_experts % count != 0 or not 1 <= keep <= count or spec.top > keep * (spec.n_experts // count):
                 raise ConfigError(f"{spec.n_experts} experts in {count} groups of which {keep} are kept do not allow "
                                   f"{spec.top} choices")
+        self.weighting = getattr(spec, "weighting", "softmax_all")
+        if self.weighting not in ("softmax_all", "softmax_chosen"):
+            raise ConfigError(f"unknown weighting of the chosen experts {self.weighting!r}; known: softmax_all, softmax_chosen")
+        if self.weighting == "softmax_chosen" and spec.groups is not None:
+            raise ConfigError("the softmax over the chosen logits alone goes without groups of experts")
+        self.router_bias = bool(getattr(spec, "router_bias", False))
         self.spec = spec
         self.dtype = ctx.dtype
         self.w_router: Optional[torch.Tensor] = None
+        self.b_router: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         s = self.spec
         specs = {"router.weight": ParamSpec((s.n_experts, s.hidden))}
+        if self.router_bias:
+            specs["router.bias"] = ParamSpec((s.n_experts,), role="gain", init="normal")
         for e in range(s.n_experts):
             specs[f"experts.{e}.gate_proj.weight"] = ParamSpec((s.intermediate, s.hidden))
             specs[f"experts.{e}.up_proj.weight"] = ParamSpec((s.intermediate, s.hidden))
@@ -54,6 +63,8 @@ class RoutedExperts(FeedForward):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.spec.n_experts
         self.w_router = tensors["router.weight"]
+        if self.router_bias:
+            self.b_router = tensors["router.bias"]
         # one tensor per kind, expert after expert: a launch reaches every expert's matrix by a stride
         self.w_gate = torch.stack([tensors[f"experts.{e}.gate_proj.weight"] for e in range(n)]).contiguous()
         self.w_up = torch.stack([tensors[f"experts.{e}.up_proj.weight"] for e in range(n)]).contiguous()
@@ -77,7 +88,12 @@ class RoutedExperts(FeedForward):
         ops.gemm(xn, self.w_router, logits, workspace=ws.scratch())
         chosen = ws.get("moe.chosen", (n, s.top), torch.int32)
         weight = ws.get("moe.weight", (n, s.top), torch.float32)
-        ops.moe_route(logits, s.top, s.groups, s.sum_eps, chosen, weight)
+        if self.b_router is not None:
+            ops.add_row_vector(logits, self.b_router)
+        # The softmax over the chosen logits alone is the softmax over all of them divided by the chosen ones' sum
+        # (the largest logit is among the chosen, so no term underflows that the other form keeps): the same kernel
+        # with nothing under the sum.
+        ops.moe_route(logits, s.top, s.groups, 0.0 if self.weighting == "softmax_chosen" else s.sum_eps, chosen, weight)
         pairs = n * s.top
         plan = ops.moe_plan(chosen, s.n_experts, ws.get("moe.plan", (ops.moe_plan_words(pairs, s.n_experts),), torch.int32))
         h = ws.get("moe.h", (pairs, s.intermediate), self.dtype)
