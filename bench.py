@@ -2,7 +2,7 @@
 """Decode and prefill speed of the Qwen3 shapes with random bfloat16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-8b|qwen3-14b|qwen3-32b]
-    python bench.py --design dokulix|felovik [--design-size 2b|8b] [--layers N]
+    python bench.py --design dokulix|felovik|sogavik [--design-size 2b|8b] [--layers N]
 
 The default run is the Qwen3-8B shape.  A step is one decode step of a batch of 8 sequences,
 each with a 2,048-token random prompt in the cache (context length 4,096): the engine's step
@@ -29,6 +29,10 @@ of launch its time against its analytical minimum (``efficiency``), from launch-
 ``--design felovik`` does the same for a Felovik model (in every layer a gated attention and a
 state-space recurrence on the same input, norms after the sums; dense feed-forwards and routed experts
 in turn, four of 32 experts a token, as many active feed-forward weights as the dense layer has).
+``--design sogavik`` measures a Sogavik model (windowed attention with a gate per head; in every second layer
+a windowed attention beside a matrix memory; routed experts and a token-side input in every layer, norms on the
+sublayers' outputs) beside the Felovik model of the same sizes, the library's closest design (a pair of mixers
+with a recurrence, routed experts).
 
 The workloads follow the reference's bench (rocml-cli/src/cmd_bench.rs:79-243): synthetic
 prompts, greedy, no stop token, warm-up first; times are taken around synchronised steps.
@@ -72,9 +76,16 @@ def felovik_config(z: dict, n_layers: int):
             "layers": [{"type": "parallel", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe} for i in range(n_layers)]}
 
 
+COMPANION = {"dokulix": "qwen3", "felovik": "qwen3", "sogavik": "felovik"}     # the closest model each design is measured beside
+
+
 def design_configs(size: dict, n_layers: int, design: str = "dokulix"):
-    """config.json of the design's model and of the Qwen3 model of equal size."""
+    """config.json of the design's model and of its companion of equal size."""
     z = size
+    if design == "sogavik":
+        from rocml_amd.config.catalog import sogavik_config
+        return (sogavik_config(z["vocab"], z["width"], z["heads"], z["kv_heads"], z["dim"], z["window"], z["width"] // 128, 128,
+                               32, z["ff"] // 4, 4, 64, n_layers, parallel_every=2), felovik_config(z, n_layers))
     att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
            "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
                      "mask": {"size": z["chunk"]}, "scale": z["dim"] ** -0.5}}
@@ -112,7 +123,8 @@ def run_design(args) -> int:
     rng = np.random.default_rng(0)
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     results = {}
-    for name, raw in zip((args.design, "qwen3"), design_configs(DESIGN_SIZES[args.design_size], n_layers, args.design)):
+    other_name = COMPANION[args.design]
+    for name, raw in zip((args.design, other_name), design_configs(DESIGN_SIZES[args.design_size], n_layers, args.design)):
         model = random_model(raw, seed=0, dtype=args.dtype, device="cuda:0")
         vocab = model.spec.vocab
         engine = Engine(model, max_tokens=batch * CONTEXT, max_seqs=batch, max_step_tokens=8192)
@@ -155,17 +167,17 @@ def run_design(args) -> int:
                          "params_m": round(model.n_params() / 1e6, 1), "launches": rows}
         del engine, model, gen
         torch.cuda.empty_cache()
-    mine, other = results[args.design], results["qwen3"]
-    out = {"metric": f"{args.design} beside the Qwen3 shape of equal size ({args.design_size}, {n_layers} layers, "
+    mine, other = results[args.design], results[other_name]
+    out = {"metric": f"{args.design} beside the {other_name} shape of equal size ({args.design_size}, {n_layers} layers, "
                      f"{args.dtype}): decode tok/s at batch {batch} over {PROMPT_LEN}-token prompts",
            "value": mine["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
            "ms_per_step": mine["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic: uniform random token ids, random N(0, 0.02) weights",
            "config": dict(DESIGN_SIZES[args.design_size], layers=n_layers, global_batch=batch, prompt_len=PROMPT_LEN),
-           "decode_vs_qwen3": round(mine["decode_tok_s"] / other["decode_tok_s"], 3),
-           "prefill_vs_qwen3": round(mine["prefill_tok_s"] / other["prefill_tok_s"], 3),
-           args.design: mine, "qwen3": other}
+           f"decode_vs_{other_name}": round(mine["decode_tok_s"] / other["decode_tok_s"], 3),
+           f"prefill_vs_{other_name}": round(mine["prefill_tok_s"] / other["prefill_tok_s"], 3),
+           args.design: mine, other_name: other}
     print(json.dumps(out))
     return 0
 
@@ -181,7 +193,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points")
     ap.add_argument("--prefill-runs", type=int, default=3)
-    ap.add_argument("--design", default=None, choices=["dokulix", "felovik"],
+    ap.add_argument("--design", default=None, choices=["dokulix", "felovik", "sogavik"],
                     help="measure this architecture at real layer sizes beside the closest Qwen3 shape, instead of the default workload")
     ap.add_argument("--design-size", default="2b", choices=sorted(DESIGN_SIZES), help="layer sizes for --design")
     ap.add_argument("--skip-prompts", action="store_true",

@@ -114,6 +114,40 @@ CATALOG += [
     ModelEntry("felovik-2b", felovik_config(32768, 2048, 16, 8, 128, 32, 64, 128, 8, 6144, 32, 1024, 4, 24)),
 ]
 
+
+
+def sogavik_config(vocab, width, heads, kv_heads, dim, window, mem_heads, mem_dim, experts, expert_ff, top, side_dim, n_layers,
+                   parallel_every=4, max_positions=40960):
+    """A Sogavik configuration: windowed attention with a gate per head in most layers (its rotation's
+    frequencies stretched fourfold beyond 4,096 positions), and in every ``parallel_every``-th layer (the third
+    among them) a windowed attention of a quarter of the window beside a matrix memory; routed experts in every
+    layer, and ``side_dim`` columns of the side table for each."""
+    def attention(w, stretched):
+        rot = {"base": 1000000.0, "dims": dim}
+        if stretched:
+            rot["scaling"] = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+        return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": w}, "rot": rot}
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}
+    layers = []
+    for i in range(n_layers):
+        if i % parallel_every == min(2, parallel_every - 1):
+            mixer = {"left": attention(max(window // 4, 1), False),
+                     "right": {"heads": mem_heads, "dim": mem_dim, "vdim": mem_dim, "gate_cap": 15.0}}
+            layers.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+        else:
+            layers.append({"type": "attention", "mixer": attention(window, True), "mlp": mlp})
+    return {"architecture": "Sogavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "token_side": {"dim": side_dim},
+            "max_positions": max_positions, "layers": layers}
+
+
+# The fourth architecture: a test-sized model and the layer sizes of a 2B-class model (random weights; no
+# checkpoint of this design exists).
+CATALOG += [
+    ModelEntry("sogavik-tiny", sogavik_config(320, 96, 4, 2, 32, 40, 2, 24, 8, 48, 2, 8, 4, max_positions=512),
+               default_ctx=512, init_norm_jitter=True),
+    ModelEntry("sogavik-2b", sogavik_config(32768, 2048, 16, 8, 128, 1024, 16, 128, 32, 1024, 4, 64, 24)),
+]
+
 _BY_NAME = {e.name: e for e in CATALOG}
 
 

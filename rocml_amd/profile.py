@@ -122,7 +122,21 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "latent_window_plan": ("expanded prompt: plan of the visible rows", _tensor_args_cost(skip=(2,))),
     "latent_window_gather": ("expanded prompt: gather of the visible rows", lambda cache, plan, out: (2 * _nbytes(out), 0)),
     "gate_heads": ("output gate", lambda x, x_stride, gate, out, n_heads, n: (2 * _nbytes(out) + out.numel() * 4, 4 * out.numel())),
-    "sigmoid_gate": ("output gate", lambda y, gate: (2 * _nbytes(y) + y.numel() * 4, 4 * y.numel())),
+    "sigmoid_gate": ("output gate", lambda y, gate, **kw: (2 * _nbytes(y) + gate.numel() * 4, 4 * y.numel())),
+    "qk_span_stats": ("q/k norm factors", lambda qkv, q_width, k_width, bias, eps, out: (
+        qkv.shape[0] * (q_width + k_width) * qkv.element_size() + _nbytes(out), 2 * qkv.shape[0] * (q_width + k_width))),
+    "norm_add": ("sublayer norm and residual sum", lambda x, y, gain, bias, eps, **kw: (
+        2 * _nbytes(x) + _nbytes(y, kw.get("copy")), 8 * x.numel())),
+    "layernorm": ("layer norm", lambda x, gain, bias, eps, out, rows=None: (out.numel() * 4 + _nbytes(out), 8 * out.numel())),
+    "token_side_gate": ("token-side gate", lambda g, table, ids, col0, out, *a, **kw: (
+        _nbytes(g, out, ids) + out.numel() * table.element_size(), 10 * out.numel())),
+    "mlstm_scan": ("matrix memory (32-bit vector work)", lambda proj, q0, k0, v0, i0, f0, ib, fb, cap, qs, fl, s_state, n_state, m_state, cu, slots,
+                   out, n_heads, head_dim, v_head_dim: (
+                       proj.shape[0] * n_heads * (2 * head_dim + v_head_dim + 2) * 4 + _nbytes(out)
+                       + 2 * slots.numel() * n_heads * head_dim * (v_head_dim + 1) * 4,
+                       4 * proj.shape[0] * n_heads * head_dim * (v_head_dim + 1), PEAK_FLOPS[torch.float32])),
+    "head_norm_gate": ("head norm and gate", lambda o, g, g_col0, gain, out, n_heads, eps: (
+        2 * _nbytes(o) + _nbytes(out), 8 * o.numel())),
     "splitk_reduce": ("sum of K pieces", _tensor_args_cost()),
     "sum_norm": ("residual sum and norm", lambda x, branches, gains, gain, eps, **kw: (
         2 * _nbytes(x) + _nbytes(*branches) + _nbytes(kw.get("copy")), 4 * x.numel() * (1 + len(branches)))),
