@@ -31,7 +31,8 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 
 __global__ void __launch_bounds__(RT_BLOCK)
 moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, int top, int group_count, int group_keep,
-                 float sum_eps, int* __restrict__ chosen, float* __restrict__ weight) {
+                 float sum_eps, int* __restrict__ chosen, float* __restrict__ weight, const float* __restrict__ bias) {
+    // bias (may be null): one number per expert, added to the logits first
     extern __shared__ float rt_smem[];          // [waves][n_experts]
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     int t = blockIdx.x * (RT_BLOCK / WAVE) + wave;
@@ -43,7 +44,7 @@ moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, 
 #pragma unroll
     for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
         int e = lane + j * WAVE;
-        s[j] = e < n_experts ? z[e] : -INFINITY;
+        s[j] = e < n_experts ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
         m = fmaxf(m, s[j]);
     }
     m = wave_max(m);
@@ -128,7 +129,7 @@ moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, 
 }
 
 ROCML_EXPORT int rocml_moe_route(const float* logits, int n_tokens, int n_experts, int top, int group_count, int group_keep,
-                                 float sum_eps, int* chosen, float* weight, hipStream_t stream) {
+                                 float sum_eps, int* chosen, float* weight, const float* bias, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && n_experts > 0 && n_experts <= RT_MAX_PER_LANE * WAVE, "moe_route: %d experts (1 to %d)", n_experts,
                   RT_MAX_PER_LANE * WAVE);
     ROCML_REQUIRE(top >= 1 && top <= WAVE && top <= n_experts, "moe_route: %d chosen of %d experts", top, n_experts);
@@ -139,7 +140,7 @@ ROCML_EXPORT int rocml_moe_route(const float* logits, int n_tokens, int n_expert
     if (n_tokens == 0) return 0;
     size_t lds = (size_t)(RT_BLOCK / WAVE) * n_experts * sizeof(float);
     moe_route_kernel<<<ceil_div(n_tokens, RT_BLOCK / WAVE), RT_BLOCK, lds, stream>>>(logits, n_tokens, n_experts, top, group_count,
-                                                                                     group_keep, sum_eps, chosen, weight);
+                                                                                     group_keep, sum_eps, chosen, weight, bias);
     ROCML_CHECK_LAUNCH("moe_route");
     return 0;
 }

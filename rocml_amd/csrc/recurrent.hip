@@ -552,11 +552,15 @@ ROCML_EXPORT int rocml_ssd_scan(const float* xbc, int ldx, const float* dtsrc, i
 // the same launch).  State layouts: S [slot, H, dv, dk] (a column's dk entries side by side), n [slot, H, tiles, dk],
 // m [slot, H, tiles], tiles = ceil(dv / SC_PT); all zero when a sequence starts.  A step of one token per sequence
 // and a step of a prompt run the same arithmetic per token.
-constexpr int ML_TC = 32;
-
 __device__ __forceinline__ float rc_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int NI>
+// VEC (rows of the projection, the columns' first numbers and the sizes are multiples of 4 numbers): a chunk's
+// operands are asked for as 16-byte pieces, all at once, while the chunk before it is worked on, and reach LDS when
+// that is done.  U tokens are worked on at a time: their operands are all read from LDS first and their sums across
+// lanes run side by side; the gates' recurrence (m, and the two factors of every token) runs ahead of them in
+// every thread.  A token past the chunk's end has keys of zero, a forget gate of one and an input gate of zero
+// (log gates 0 and -infinity): it leaves S, n and m as they are, bit for bit.
+template <int NI, bool VEC>
 __global__ void __launch_bounds__(RC_BLOCK)
 mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0, int v_col0, int i_col0, int f_col0,
                   const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale, float floor_,
@@ -565,11 +569,13 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
                   int n_heads, int dk, int dv, int tiles) {
     extern __shared__ float4 ml_smem4[];
     constexpr int NP = SC_R * NI;              // padded length of a q or k row
-    float* ks = (float*)ml_smem4;              // [ML_TC][NP]
-    float* qs = ks + ML_TC * NP;               // [ML_TC][NP]
-    float* vs = qs + ML_TC * NP;               // [ML_TC][SC_PT]
-    float* os = vs + ML_TC * SC_PT;            // [ML_TC][SC_PT]
-    float* gs = os + ML_TC * SC_PT;            // [ML_TC][2]: log input gate, log forget gate
+    constexpr int TC = NI <= 8 ? 32 : 16;      // tokens of a chunk
+    constexpr int U = NI <= 8 ? 4 : 2;         // tokens worked on at a time
+    float* ks = (float*)ml_smem4;              // [TC][NP]
+    float* qs = ks + TC * NP;                  // [TC][NP]
+    float* vs = qs + TC * NP;                  // [TC][SC_PT]
+    float* os = vs + TC * SC_PT;               // [TC][SC_PT]
+    float* gs = os + TC * SC_PT;               // [TC][2]: log input gate, log forget gate
     int tile = blockIdx.x, p0 = tile * SC_PT, head = blockIdx.y, b = blockIdx.z;
     int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
     int first = cu_seqlens[b], n_tok = cu_seqlens[b + 1] - first;
@@ -585,61 +591,129 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
     sc_load_state<NI>(nn, n_mine, r, dk, true);
     float m = m_state[slot_head * tiles + tile];
     float bi = i_bias ? i_bias[head] : 0.f, bf = f_bias ? f_bias[head] : 0.f;
-    for (int c0 = 0; c0 < n_tok; c0 += ML_TC) {
-        int nt = min(ML_TC, n_tok - c0);
+    constexpr int PF = VEC ? (TC * NP / 4 + RC_BLOCK - 1) / RC_BLOCK : 1;
+    sc_f4 pre_k[PF], pre_q[PF], pre_v;
+    float pre_i = 0.f, pre_f = 0.f;
+    const sc_f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    pre_v = zero4;
+#define ML_PREFETCH(c0_)                                                                                         \
+    {                                                                                                            \
+        int nt_ = min(TC, n_tok - (c0_));                                                                        \
+        _Pragma("unroll") for (int j = 0; j < PF; ++j) {                                                         \
+            int i4 = tid + j * RC_BLOCK, tt = i4 / (NP / 4), d = (i4 - tt * (NP / 4)) * 4;                       \
+            bool ok = tt < nt_ && d < dk;                                                                        \
+            const float* row = proj + (size_t)(first + (c0_) + (ok ? tt : 0)) * ld + (size_t)head * dk + (ok ? d : 0); \
+            pre_k[j] = ok ? *(const sc_f4*)(row + k_col0) : zero4;                                              \
+            pre_q[j] = ok ? *(const sc_f4*)(row + q_col0) : zero4;                                              \
+        }                                                                                                        \
+        {                                                                                                        \
+            int tt = tid / (SC_PT / 4), pp = (tid - tt * (SC_PT / 4)) * 4;                                       \
+            bool ok = tt < nt_ && p0 + pp < dv;                                                                  \
+            pre_v = ok ? *(const sc_f4*)(proj + (size_t)(first + (c0_) + tt) * ld + v_col0 + (size_t)head * dv + p0 + pp) : zero4; \
+        }                                                                                                        \
+        if (tid < nt_) {                                                                                         \
+            const float* row = proj + (size_t)(first + (c0_) + tid) * ld;                                        \
+            pre_i = row[i_col0 + head];                                                                          \
+            pre_f = row[f_col0 + head];                                                                          \
+        }                                                                                                        \
+    }
+    if (VEC && n_tok > 0) ML_PREFETCH(0)
+    for (int c0 = 0; c0 < n_tok; c0 += TC) {
+        int nt = min(TC, n_tok - c0);
+        int nt_up = (nt + U - 1) / U * U;
         __syncthreads();                          // the previous chunk's outputs have been written out
-        for (int i = tid; i < nt * NP; i += RC_BLOCK) {
-            int tt = i / NP, d = i - tt * NP;
-            const float* row = proj + (size_t)(first + c0 + tt) * ld + (size_t)head * dk + d;
-            bool ok = d < dk;
-            ks[i] = ok ? row[k_col0] : 0.f;
-            qs[i] = ok ? row[q_col0] * q_scale : 0.f;
-        }
-        for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
-            int tt = i / SC_PT, pp = i - tt * SC_PT;
-            vs[i] = p0 + pp < dv ? proj[(size_t)(first + c0 + tt) * ld + v_col0 + (size_t)head * dv + p0 + pp] : 0.f;
-        }
-        if (tid < nt) {
-            const float* row = proj + (size_t)(first + c0 + tid) * ld;
-            gs[2 * tid] = cap * tanhf((row[i_col0 + head] + bi) / cap);
-            gs[2 * tid + 1] = rc_logsigmoid(cap * tanhf((row[f_col0 + head] + bf) / cap));
-        }
-        __syncthreads();
-        for (int tt = 0; tt < nt; ++tt) {
-            float2 g = *(const float2*)(gs + 2 * tt);
-            float2 xv = *(const float2*)(vs + tt * SC_PT + pl * SC_PP);
-            float kv[NI], qv[NI];
-            const float* kt = ks + tt * NP + r * NI;
-            const float* qt = qs + tt * NP + r * NI;
-            if (NI % 4 == 0) {
+        if (VEC) {
 #pragma unroll
-                for (int i = 0; i < NI; i += 4) {
-                    float4 k4 = *(const float4*)(kt + i), q4 = *(const float4*)(qt + i);
-                    kv[i] = k4.x; kv[i + 1] = k4.y; kv[i + 2] = k4.z; kv[i + 3] = k4.w;
-                    qv[i] = q4.x; qv[i + 1] = q4.y; qv[i + 2] = q4.z; qv[i + 3] = q4.w;
+            for (int j = 0; j < PF; ++j) {
+                int i4 = tid + j * RC_BLOCK;
+                if (i4 < TC * (NP / 4)) {
+                    ((sc_f4*)ks)[i4] = pre_k[j];
+                    ((sc_f4*)qs)[i4] = pre_q[j] * q_scale;
                 }
-            } else {
-#pragma unroll
-                for (int i = 0; i < NI; ++i) { kv[i] = kt[i]; qv[i] = qt[i]; }
             }
-            float m_new = fmaxf(g.y + m, g.x);
-            float a = expf(g.y + m - m_new), bb = expf(g.x - m_new);
-            m = m_new;
-            float bv0 = bb * xv.x, bv1 = bb * xv.y, q0 = 0.f, q1 = 0.f, nq = 0.f;
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                s[0][i] = fmaf(a, s[0][i], bv0 * kv[i]);
-                s[1][i] = fmaf(a, s[1][i], bv1 * kv[i]);
-                nn[i] = fmaf(a, nn[i], bb * kv[i]);
-                q0 = fmaf(s[0][i], qv[i], q0);
-                q1 = fmaf(s[1][i], qv[i], q1);
-                nq = fmaf(nn[i], qv[i], nq);
+            if (tid < TC * (SC_PT / 4)) ((sc_f4*)vs)[tid] = pre_v;
+            if (tid < TC) {
+                gs[2 * tid] = tid < nt ? cap * tanhf((pre_i + bi) / cap) : -INFINITY;
+                gs[2 * tid + 1] = tid < nt ? rc_logsigmoid(cap * tanhf((pre_f + bf) / cap)) : 0.f;
             }
-            q0 = row16_sum(q0);
-            q1 = row16_sum(q1);
-            nq = row16_sum(nq);
-            float den = fmaxf(fabsf(nq), expf(-m)) + floor_;
-            if (r == 0) *(float2*)(os + tt * SC_PT + pl * SC_PP) = make_float2(q0 / den, q1 / den);
+            __syncthreads();
+            if (c0 + TC < n_tok) ML_PREFETCH(c0 + TC)
+        } else {
+            for (int i = tid; i < nt_up * NP; i += RC_BLOCK) {
+                int tt = i / NP, d = i - tt * NP;
+                bool ok = tt < nt && d < dk;
+                const float* row = proj + (size_t)(first + c0 + (ok ? tt : 0)) * ld + (size_t)head * dk + (ok ? d : 0);
+                ks[i] = ok ? row[k_col0] : 0.f;
+                qs[i] = ok ? row[q_col0] * q_scale : 0.f;
+            }
+            for (int i = tid; i < nt_up * SC_PT; i += RC_BLOCK) {
+                int tt = i / SC_PT, pp = i - tt * SC_PT;
+                vs[i] = (tt < nt && p0 + pp < dv) ? proj[(size_t)(first + c0 + tt) * ld + v_col0 + (size_t)head * dv + p0 + pp] : 0.f;
+            }
+            if (tid < nt_up) {
+                const float* row = proj + (size_t)(first + c0 + min(tid, nt - 1)) * ld;
+                gs[2 * tid] = tid < nt ? cap * tanhf((row[i_col0 + head] + bi) / cap) : -INFINITY;
+                gs[2 * tid + 1] = tid < nt ? rc_logsigmoid(cap * tanhf((row[f_col0 + head] + bf) / cap)) : 0.f;
+            }
+            __syncthreads();
+        }
+        for (int t0 = 0; t0 < nt; t0 += U) {
+            float2 xv[U];
+            float kv[U][NI], qv[U][NI], fa[U], fb[U], em[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                int tt = t0 + u;
+                float2 g = *(const float2*)(gs + 2 * tt);
+                float m_new = fmaxf(g.y + m, g.x);
+                fa[u] = expf(g.y + m - m_new);
+                fb[u] = expf(g.x - m_new);
+                m = m_new;
+                em[u] = expf(-m);
+                xv[u] = *(const float2*)(vs + tt * SC_PT + pl * SC_PP);
+                const float* kt = ks + tt * NP + r * NI;
+                const float* qt = qs + tt * NP + r * NI;
+                if (NI % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < NI; i += 4) {
+                        float4 k4 = *(const float4*)(kt + i), q4 = *(const float4*)(qt + i);
+                        kv[u][i] = k4.x; kv[u][i + 1] = k4.y; kv[u][i + 2] = k4.z; kv[u][i + 3] = k4.w;
+                        qv[u][i] = q4.x; qv[u][i + 1] = q4.y; qv[u][i + 2] = q4.z; qv[u][i + 3] = q4.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NI; ++i) { kv[u][i] = kt[i]; qv[u][i] = qt[i]; }
+                }
+            }
+            float part0[U], part1[U], partn[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float a = fa[u], bb = fb[u], bv0 = bb * xv[u].x, bv1 = bb * xv[u].y, q0 = 0.f, q1 = 0.f, nq = 0.f;
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    s[0][i] = fmaf(a, s[0][i], bv0 * kv[u][i]);
+                    s[1][i] = fmaf(a, s[1][i], bv1 * kv[u][i]);
+                    nn[i] = fmaf(a, nn[i], bb * kv[u][i]);
+                    q0 = fmaf(s[0][i], qv[u][i], q0);
+                    q1 = fmaf(s[1][i], qv[u][i], q1);
+                    nq = fmaf(nn[i], qv[u][i], nq);
+                }
+                part0[u] = q0;
+                part1[u] = q1;
+                partn[u] = nq;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                part0[u] = row16_sum(part0[u]);
+                part1[u] = row16_sum(part1[u]);
+                partn[u] = row16_sum(partn[u]);
+            }
+            if (r == 0) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float den = fmaxf(fabsf(partn[u]), em[u]) + floor_;
+                    *(float2*)(os + (t0 + u) * SC_PT + pl * SC_PP) = make_float2(part0[u] / den, part1[u] / den);
+                }
+            }
         }
         __syncthreads();
         for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
@@ -647,6 +721,7 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
             if (p0 + pp < dv) out[(size_t)(first + c0 + tt) * n_heads * dv + (size_t)head * dv + p0 + pp] = os[i];
         }
     }
+#undef ML_PREFETCH
 #pragma unroll
     for (int j = 0; j < SC_PP; ++j) {
         int p = p0 + pl * SC_PP + j;
@@ -677,11 +752,22 @@ ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_c
     dim3 grid(tiles, n_heads, n_seqs);
     int ni = ceil_div(dk, SC_R);
     ni = ni <= 4 ? ni : ni <= 6 ? 6 : ni <= 8 ? 8 : ni <= 12 ? 12 : 16;
-    size_t lds = (size_t)(2 * ML_TC * SC_R * ni + 2 * ML_TC * SC_PT + 2 * ML_TC) * sizeof(float);
+    int tc = ni <= 8 ? 32 : 16;
+    size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
+    // whole 16-byte pieces: every row of q, k and v starts on a multiple of 4 numbers and ends on one
+    bool vec = ld % 4 == 0 && dk % 4 == 0 && dv % 4 == 0 && q_col0 % 4 == 0 && k_col0 % 4 == 0 && v_col0 % 4 == 0 &&
+               ((uintptr_t)proj & 15) == 0;
 #define MSCAN(NI_)                                                                                                     \
-    mlstm_scan_kernel<NI_><<<grid, RC_BLOCK, lds, stream>>>(proj, ld, q_col0, k_col0, v_col0, i_col0, f_col0, i_bias, f_bias, \
-                                                            cap, q_scale, floor_, s_state, n_state, m_state, cu_seqlens,  \
-                                                            seq_slots, out, n_heads, dk, dv, tiles)
+    {                                                                                                                  \
+        if (vec)                                                                                                       \
+            mlstm_scan_kernel<NI_, true><<<grid, RC_BLOCK, lds, stream>>>(proj, ld, q_col0, k_col0, v_col0, i_col0, f_col0, i_bias, \
+                                                                          f_bias, cap, q_scale, floor_, s_state, n_state, m_state, \
+                                                                          cu_seqlens, seq_slots, out, n_heads, dk, dv, tiles);  \
+        else                                                                                                           \
+            mlstm_scan_kernel<NI_, false><<<grid, RC_BLOCK, lds, stream>>>(proj, ld, q_col0, k_col0, v_col0, i_col0, f_col0, i_bias, \
+                                                                           f_bias, cap, q_scale, floor_, s_state, n_state, m_state, \
+                                                                           cu_seqlens, seq_slots, out, n_heads, dk, dv, tiles); \
+    }
     switch (ni) {
         case 1: MSCAN(1); break;
         case 2: MSCAN(2); break;

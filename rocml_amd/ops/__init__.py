@@ -57,7 +57,7 @@ _SIGNATURES = {
         "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
     },
     "moe": {
-        "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+        "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P, _P],
         "rocml_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _I, _P],
         "rocml_moe_gemm": [_P, _I, _I, _I, _P, _I, _P, _P, _I, _LL, _I, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
         "rocml_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
@@ -1151,12 +1151,15 @@ def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
     return max(1, min(n_pairs, n_pairs // MOE_TILE_ROWS + n_experts))
 
 
-def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: torch.Tensor, weight: torch.Tensor) -> None:
+def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: torch.Tensor, weight: torch.Tensor,
+              bias: Optional[torch.Tensor] = None) -> None:
     """Softmax over all experts, the ``top`` best (of the experts of the ``groups[1]`` best of
     ``groups[0]`` equal groups of neighbours, a group's score being its largest, if ``groups`` is
     given), weights = chosen scores / (their sum + ``sum_eps``).  ``chosen`` int32, ``weight`` float32,
-    both ``[T, top]``."""
-    _dev(logits, chosen, weight)
+    both ``[T, top]``.  ``bias``: 32-bit, one number per expert, added to the logits first."""
+    _dev(logits, chosen, weight, bias)
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != logits.shape[1]):
+        raise KernelError("the router's bias must be 32-bit with one number per expert")
     _want(logits, torch.float32, "router logits")
     _want(chosen, torch.int32, "chosen experts")
     _want(weight, torch.float32, "expert weights")
@@ -1165,7 +1168,7 @@ def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: to
         raise KernelError("moe_route: outputs must be [tokens, top]")
     count, keep = (0, 0) if groups is None else (int(groups[0]), int(groups[1]))
     _check("moe", library("moe").rocml_moe_route(_ptr(logits), n_tokens, n_experts, top, count, keep, float(sum_eps),
-                                                 _ptr(chosen), _ptr(weight), _stream()))
+                                                 _ptr(chosen), _ptr(weight), _ptr(bias), _stream()))
 
 
 def moe_plan(chosen: torch.Tensor, n_experts: int, plan: torch.Tensor):

@@ -88,12 +88,11 @@ class RoutedExperts(FeedForward):
         ops.gemm(xn, self.w_router, logits, workspace=ws.scratch())
         chosen = ws.get("moe.chosen", (n, s.top), torch.int32)
         weight = ws.get("moe.weight", (n, s.top), torch.float32)
-        if self.b_router is not None:
-            ops.add_row_vector(logits, self.b_router)
         # The softmax over the chosen logits alone is the softmax over all of them divided by the chosen ones' sum
         # (the largest logit is among the chosen, so no term underflows that the other form keeps): the same kernel
         # with nothing under the sum.
-        ops.moe_route(logits, s.top, s.groups, 0.0 if self.weighting == "softmax_chosen" else s.sum_eps, chosen, weight)
+        ops.moe_route(logits, s.top, s.groups, 0.0 if self.weighting == "softmax_chosen" else s.sum_eps, chosen, weight,
+                      bias=self.b_router)
         pairs = n * s.top
         plan = ops.moe_plan(chosen, s.n_experts, ws.get("moe.plan", (ops.moe_plan_words(pairs, s.n_experts),), torch.int32))
         h = ws.get("moe.h", (pairs, s.intermediate), self.dtype)

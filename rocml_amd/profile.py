@@ -148,7 +148,7 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
                                      4 * xbc.shape[0] * n_heads * head_dim * n_state, PEAK_FLOPS[torch.float32])),
     "gated_part_norm": ("gated norm in parts", lambda y, z, z_col0, gain, out, parts, eps: (
         2 * _nbytes(y) + _nbytes(out), 8 * y.numel())),
-    "moe_route": ("choice of experts", lambda logits, top, groups, sum_eps, chosen, weight: (_nbytes(logits, chosen, weight),
+    "moe_route": ("choice of experts", lambda logits, top, groups, sum_eps, chosen, weight, **kw: (_nbytes(logits, chosen, weight),
                                                                                             4 * logits.numel())),
     "moe_plan": ("plan of the experts' rows", lambda chosen, n_experts, plan: (3 * _nbytes(chosen), 0)),
     "moe_gemm": ("experts' products", lambda a, w, out, plan, top, gather, w2=None, **kw: (
