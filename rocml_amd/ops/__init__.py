@@ -305,7 +305,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     n_tokens, ld = qkv.shape
     if bias is not None:
         _want(bias, torch.float32, "projection bias")
-        if bias.numel() != ld:
+        # (rows may be wider than the projection: a product shared with other mixers, whose columns follow)
+        if bias.numel() > ld or bias.numel() < n_heads * head_dim + (n_kv_heads * (head_dim + dv) if write_kv else 0):
             raise KernelError(f"the bias has {bias.numel()} values for rows of {ld}")
     if span_inv is not None:
         _want(span_inv, torch.float32, "norm factors")
@@ -939,15 +940,11 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
     if v_cache.dtype != k_cache.dtype or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
             or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
         raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
-    if span_inv is not None:
-        _want(span_inv, torch.float32, "norm factors")
-        if span_inv.shape != (n_tokens, 2) or n_splits > 1 or q_gain is None or k_gain is None:
-            raise KernelError("a norm over the whole projection needs [tokens, 2] factors, a complete projection and both gains")
-    for g, heads in ((q_gain, n_heads), (k_gain, n_kv_heads)):
+    for g in (q_gain, k_gain):
         if g is not None:
             _want(g, torch.float32, "head norm gain")
-            if g.numel() != (head_dim if span_inv is None else heads * head_dim):
-                raise KernelError(f"norm gain has {g.numel()} values for {heads} heads of size {head_dim}")
+            if g.numel() != head_dim:
+                raise KernelError(f"head norm gain has {g.numel()} values for head size {head_dim}")
     if cos is not None:
         _want(cos, torch.float32, "rotation table")
         if cos.shape != (n_tokens, head_dim // 2) or sin is None or sin.shape != cos.shape or sin.dtype != cos.dtype:

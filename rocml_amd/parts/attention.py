@@ -188,7 +188,7 @@ class Attention(Mixer):
     def input_weight(self) -> Optional[torch.Tensor]:
         # only the path of the norm-and-rotation kernel, which takes rows of any stride; and the
         # projection must start at the buffer's first column
-        return self.w_qkv if self.separate_q and not self.spec.bias else None
+        return self.w_qkv if self.separate_q else None
 
     def adopt_input_weight(self, view: torch.Tensor) -> None:
         self.w_qkv = view
