@@ -666,27 +666,61 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
 
 // ---- factors of a norm over a token's whole q row and whole k row ---------------------------
 // inv[t, 0] = 1 / sqrt(mean over the q_width leading columns of (row + bias)^2 + eps), inv[t, 1] the same over the
-// k_width columns behind them.  One block per token; 32-bit.
+// k_width columns behind them.  One wave per token; 32-bit.
 template <typename TI>
 __global__ void __launch_bounds__(EW_BLOCK)
-qk_span_stats_kernel(const TI* __restrict__ qkv, int ld, int q_width, int k_width, const float* __restrict__ bias,
+qk_span_stats_kernel(const TI* __restrict__ qkv, int ld, int n_tokens, int q_width, int k_width, const float* __restrict__ bias,
                      float eps, float* __restrict__ inv) {
-    __shared__ float scratch[EW_BLOCK / WAVE];
-    const TI* row = qkv + (size_t)blockIdx.x * ld;
+    // a wave per token: no barrier, and all of a lane's loads are on their way together
+    int lane = threadIdx.x & (WAVE - 1);
+    long long t = (long long)blockIdx.x * (EW_BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (t >= n_tokens) return;
+    const TI* row = qkv + (size_t)t * ld;
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < q_width; i += EW_BLOCK) {
+    for (int i = lane; i < q_width; i += WAVE) {
         float v = Elem<TI>::load(row + i) + (bias ? bias[i] : 0.f);
         sq = fmaf(v, v, sq);
     }
-    for (int i = threadIdx.x; i < k_width; i += EW_BLOCK) {
+    for (int i = lane; i < k_width; i += WAVE) {
         float v = Elem<TI>::load(row + q_width + i) + (bias ? bias[q_width + i] : 0.f);
         sk = fmaf(v, v, sk);
     }
-    sq = block_sum(sq, scratch);
-    sk = block_sum(sk, scratch);
-    if (threadIdx.x == 0) {
-        inv[(size_t)blockIdx.x * 2] = 1.0f / sqrtf(sq / (float)q_width + eps);
-        inv[(size_t)blockIdx.x * 2 + 1] = 1.0f / sqrtf(sk / (float)k_width + eps);
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) {
+        inv[(size_t)t * 2] = 1.0f / sqrtf(sq / (float)q_width + eps);
+        inv[(size_t)t * 2 + 1] = 1.0f / sqrtf(sk / (float)k_width + eps);
+    }
+}
+
+// The same for 32-bit rows whose q and k parts are whole 16-byte pieces.
+__global__ void __launch_bounds__(EW_BLOCK)
+qk_span_stats_vec_kernel(const float* __restrict__ qkv, int ld, int n_tokens, int q_width, int k_width,
+                         const float* __restrict__ bias, float eps, float* __restrict__ inv) {
+    int lane = threadIdx.x & (WAVE - 1);
+    long long t = (long long)blockIdx.x * (EW_BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (t >= n_tokens) return;
+    const float4* row = (const float4*)(qkv + (size_t)t * ld);
+    const float4* b4 = (const float4*)bias;
+    int nq = q_width / 4, nk = k_width / 4;
+    float sq = 0.f, sk = 0.f;
+#pragma unroll 4
+    for (int i = lane; i < nq; i += WAVE) {
+        float4 v = row[i];
+        if (bias) { float4 b = b4[i]; v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w; }
+        sq = fmaf(v.x, v.x, sq); sq = fmaf(v.y, v.y, sq); sq = fmaf(v.z, v.z, sq); sq = fmaf(v.w, v.w, sq);
+    }
+#pragma unroll 4
+    for (int i = lane; i < nk; i += WAVE) {
+        float4 v = row[nq + i];
+        if (bias) { float4 b = b4[nq + i]; v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w; }
+        sk = fmaf(v.x, v.x, sk); sk = fmaf(v.y, v.y, sk); sk = fmaf(v.z, v.z, sk); sk = fmaf(v.w, v.w, sk);
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) {
+        inv[(size_t)t * 2] = 1.0f / sqrtf(sq / (float)q_width + eps);
+        inv[(size_t)t * 2 + 1] = 1.0f / sqrtf(sk / (float)k_width + eps);
     }
 }
 
@@ -695,10 +729,15 @@ ROCML_EXPORT int rocml_qk_span_stats(const void* qkv, int dtype, int ld, int n_t
     ROCML_REQUIRE(n_tokens >= 0 && q_width > 0 && k_width > 0 && ld >= q_width + k_width && qkv && inv,
                   "qk_span_stats: bad sizes T=%d q=%d k=%d ld=%d", n_tokens, q_width, k_width, ld);
     if (n_tokens == 0) return 0;
-    if (dtype == ROCML_F32)
-        qk_span_stats_kernel<float><<<n_tokens, EW_BLOCK, 0, stream>>>((const float*)qkv, ld, q_width, k_width, bias, eps, inv);
+    int grid = ceil_div(n_tokens, EW_BLOCK / WAVE);
+    bool vec = dtype == ROCML_F32 && ld % 4 == 0 && q_width % 4 == 0 && k_width % 4 == 0 && (uintptr_t)qkv % 16 == 0 &&
+               (!bias || (uintptr_t)bias % 16 == 0);
+    if (vec)
+        qk_span_stats_vec_kernel<<<grid, EW_BLOCK, 0, stream>>>((const float*)qkv, ld, n_tokens, q_width, k_width, bias, eps, inv);
+    else if (dtype == ROCML_F32)
+        qk_span_stats_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((const float*)qkv, ld, n_tokens, q_width, k_width, bias, eps, inv);
     else if (dtype == ROCML_BF16)
-        qk_span_stats_kernel<bf16_t><<<n_tokens, EW_BLOCK, 0, stream>>>((const bf16_t*)qkv, ld, q_width, k_width, bias, eps, inv);
+        qk_span_stats_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)qkv, ld, n_tokens, q_width, k_width, bias, eps, inv);
     else return rocml_fail("qk_span_stats: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("qk_span_stats");
     return 0;

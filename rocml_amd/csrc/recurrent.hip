@@ -731,6 +731,84 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
     if (tid == 0) m_state[slot_head * tiles + tile] = m;
 }
 
+// A step of one token per sequence: the same arithmetic for that token without the chunks: a thread reads its
+// entries of k and q and its two values of v straight from memory, next to its state entries, and nothing waits at
+// a barrier.  Token b is sequence b's.
+template <int NI>
+__global__ void __launch_bounds__(RC_BLOCK)
+mlstm_step_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0, int v_col0, int i_col0, int f_col0,
+                  const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale, float floor_,
+                  float* __restrict__ s_state, float* __restrict__ n_state, float* __restrict__ m_state,
+                  const int* __restrict__ seq_slots, float* __restrict__ out, int n_heads, int dk, int dv, int tiles,
+                  int vec_rows) {
+    int tile = blockIdx.x, p0 = tile * SC_PT, head = blockIdx.y, b = blockIdx.z;
+    int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
+    size_t slot_head = (size_t)seq_slots[b] * n_heads + head;
+    float* st_head = s_state + slot_head * dv * dk;
+    float* n_mine = n_state + (slot_head * tiles + tile) * dk;
+    const float* row = proj + (size_t)b * ld;
+    const float* krow = row + k_col0 + (size_t)head * dk;
+    const float* qrow = row + q_col0 + (size_t)head * dk;
+    float s[SC_PP][NI], nn[NI], kv[NI], qv[NI];
+    // (k and q are read like a column of the state; their rows start on 16 bytes where the vector form is taken:
+    // the caller checks the strides)
+    sc_load_state<NI>(kv, krow, r, vec_rows ? dk : -1, true);
+    sc_load_state<NI>(qv, qrow, r, vec_rows ? dk : -1, true);
+    if (!vec_rows) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            int d = r * NI + i;
+            bool ok = d < dk;
+            kv[i] = ok ? krow[d] : 0.f;
+            qv[i] = ok ? qrow[d] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) qv[i] *= q_scale;
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        sc_load_state<NI>(s[j], st_head + (size_t)min(p, dv - 1) * dk, r, dk, p < dv);
+    }
+    sc_load_state<NI>(nn, n_mine, r, dk, true);
+    float m = m_state[slot_head * tiles + tile];
+    float xv[SC_PP];
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        xv[j] = p < dv ? row[v_col0 + (size_t)head * dv + p] : 0.f;
+    }
+    float gi = cap * tanhf((row[i_col0 + head] + (i_bias ? i_bias[head] : 0.f)) / cap);
+    float gf = rc_logsigmoid(cap * tanhf((row[f_col0 + head] + (f_bias ? f_bias[head] : 0.f)) / cap));
+    float m_new = fmaxf(gf + m, gi);
+    float a = expf(gf + m - m_new), bb = expf(gi - m_new);
+    m = m_new;
+    float em = expf(-m);
+    float bv0 = bb * xv[0], bv1 = bb * xv[1], q0 = 0.f, q1 = 0.f, nq = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        s[0][i] = fmaf(a, s[0][i], bv0 * kv[i]);
+        s[1][i] = fmaf(a, s[1][i], bv1 * kv[i]);
+        nn[i] = fmaf(a, nn[i], bb * kv[i]);
+        q0 = fmaf(s[0][i], qv[i], q0);
+        q1 = fmaf(s[1][i], qv[i], q1);
+        nq = fmaf(nn[i], qv[i], nq);
+    }
+    q0 = row16_sum(q0);
+    q1 = row16_sum(q1);
+    nq = row16_sum(nq);
+    float den = fmaxf(fabsf(nq), em) + floor_;
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        if (p >= dv) continue;
+        if (r == 0) out[(size_t)b * n_heads * dv + (size_t)head * dv + p] = (j == 0 ? q0 : q1) / den;
+        sc_store_state<NI>(s[j], st_head + (size_t)p * dk, r, dk, true);
+    }
+    if (pl == 0) sc_store_state<NI>(nn, n_mine, r, dk, true);
+    if (tid == 0) m_state[slot_head * tiles + tile] = m;
+}
+
 ROCML_EXPORT int rocml_mlstm_tile() { return SC_PT; }
 
 ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_col0, int v_col0, int i_col0, int f_col0,
@@ -752,6 +830,27 @@ ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_c
     dim3 grid(tiles, n_heads, n_seqs);
     int ni = ceil_div(dk, SC_R);
     ni = ni <= 4 ? ni : ni <= 6 ? 6 : ni <= 8 ? 8 : ni <= 12 ? 12 : 16;
+    if (n_tokens == n_seqs) {          // one token per sequence (every sequence of a step brings at least one)
+        // k and q rows as 16-byte pieces: every row and every head's part starts on a multiple of 4 numbers
+        int vec_rows = ld % 4 == 0 && dk % 4 == 0 && q_col0 % 4 == 0 && k_col0 % 4 == 0 && ((uintptr_t)proj & 15) == 0;
+#define MSTEP(NI_)                                                                                                     \
+    mlstm_step_kernel<NI_><<<grid, RC_BLOCK, 0, stream>>>(proj, ld, q_col0, k_col0, v_col0, i_col0, f_col0, i_bias, f_bias, cap, \
+                                                          q_scale, floor_, s_state, n_state, m_state, seq_slots, out, n_heads, dk, \
+                                                          dv, tiles, vec_rows)
+        switch (ni) {
+            case 1: MSTEP(1); break;
+            case 2: MSTEP(2); break;
+            case 3: MSTEP(3); break;
+            case 4: MSTEP(4); break;
+            case 6: MSTEP(6); break;
+            case 8: MSTEP(8); break;
+            case 12: MSTEP(12); break;
+            default: MSTEP(16); break;
+        }
+#undef MSTEP
+        ROCML_CHECK_LAUNCH("mlstm_scan step");
+        return 0;
+    }
     int tc = ni <= 8 ? 32 : 16;
     size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
     // whole 16-byte pieces: every row of q, k and v starts on a multiple of 4 numbers and ends on one
@@ -806,6 +905,59 @@ head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ g, 
     }
 }
 
+__device__ __forceinline__ void rc_store4(float* p, float a, float b, float c, float d) { *(sc_f4*)p = sc_f4{a, b, c, d}; }
+__device__ __forceinline__ void rc_store4(bf16_t* p, float a, float b, float c, float d) {
+    uint2 v;
+    v.x = f32x2_to_bf16x2(a, b);
+    v.y = f32x2_to_bf16x2(c, d);
+    *(uint2*)p = v;
+}
+
+// Heads of up to 512 values that are multiples of 4, rows that start on 16 bytes: the head stays in registers as
+// 16-byte pieces between the sum and the product, and gate and gain are read the same way.
+template <typename TO>
+__global__ void __launch_bounds__(RC_BLOCK)
+head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__ g, int ldg, int g_col0,
+                          const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps) {
+    int lane = threadIdx.x & (WAVE - 1);
+    long long row = (long long)blockIdx.x * (RC_BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (row >= n_rows) return;
+    long long t = row / n_heads;
+    int h = (int)(row - t * n_heads);
+    int nv = dv / 4;
+    const sc_f4* src = (const sc_f4*)(o + (size_t)row * dv);
+    const sc_f4* gr = (const sc_f4*)(g + (size_t)t * ldg + g_col0 + (size_t)h * dv);
+    const sc_f4* wr = (const sc_f4*)(gain + (size_t)h * dv);
+    const sc_f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    sc_f4 v[2], z[2], w[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        int c = lane + k * WAVE;
+        bool ok = c < nv;
+        v[k] = ok ? src[c] : zero4;
+        z[k] = ok ? gr[c] : zero4;
+        w[k] = ok ? wr[c] : zero4;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        ss = fmaf(v[k].x, v[k].x, ss); ss = fmaf(v[k].y, v[k].y, ss);
+        ss = fmaf(v[k].z, v[k].z, ss); ss = fmaf(v[k].w, v[k].w, ss);
+    }
+    float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        int c = lane + k * WAVE;
+        if (c >= nv) continue;
+        TO* dst = out + (size_t)row * dv + 4 * (size_t)c;
+        float r0 = v[k].x * inv * w[k].x * (1.0f / (1.0f + expf(-z[k].x)));
+        float r1 = v[k].y * inv * w[k].y * (1.0f / (1.0f + expf(-z[k].y)));
+        float r2 = v[k].z * inv * w[k].z * (1.0f / (1.0f + expf(-z[k].z)));
+        float r3 = v[k].w * inv * w[k].w * (1.0f / (1.0f + expf(-z[k].w)));
+        rc_store4(dst, r0, r1, r2, r3);
+    }
+}
+
 ROCML_EXPORT int rocml_head_norm_gate(const float* o, const float* g, int ldg, int g_col0, const float* gain, void* out,
                                       int out_dtype, int n_tokens, int n_heads, int dv, float eps, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && dv > 0 && g_col0 >= 0 && ldg >= g_col0 + n_heads * dv && o && g && gain && out,
@@ -813,7 +965,13 @@ ROCML_EXPORT int rocml_head_norm_gate(const float* o, const float* g, int ldg, i
     long long rows = (long long)n_tokens * n_heads;
     if (rows == 0) return 0;
     int grid = ceil_div(rows, RC_BLOCK / WAVE);
-    if (out_dtype == ROCML_F32)
+    bool vec = dv % 4 == 0 && dv <= 8 * WAVE && ldg % 4 == 0 && g_col0 % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0 &&
+               (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0;
+    if (vec && out_dtype == ROCML_F32)
+        head_norm_gate_vec_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
+    else if (vec && out_dtype == ROCML_BF16)
+        head_norm_gate_vec_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
+    else if (out_dtype == ROCML_F32)
         head_norm_gate_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
     else if (out_dtype == ROCML_BF16)
         head_norm_gate_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
