@@ -320,9 +320,10 @@ __global__ void qk_norm_rope_append_kernel(
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
     int rows_per_token, int pairing, int first_row, const float* __restrict__ bias, int dv,
-    float qt_coef, int qt_every, const float* __restrict__ span_inv) {
+    float qt_coef, int qt_every, const float* __restrict__ span_inv, int span_self) {
     // span_inv (may be null): [T, 2], the norm's factor of a token's whole q row and whole k row; the gains then
-    // have one number per column of the q (k) projection, and a head takes its own part of them.
+    // have one number per column of the q (k) projection, and a head takes its own part of them.  span_self: the
+    // same norm, but every wave forms its row's factor itself (few tokens: one launch less).
     // qt_coef, qt_every: the queries' stretch with their position (after the norm); every = 0: none.
     // bias (may be null): one number per column of the packed row, added to the projection's sums.
     // dv: the size of a value head; the value rows start behind the Hq + Hkv rows of d numbers.
@@ -367,6 +368,29 @@ __global__ void qk_norm_rope_append_kernel(
         float inv;
         if (span_inv) {
             inv = span_inv[(size_t)t * 2 + kind];
+            gain += (size_t)(kind == 0 ? r : r - hq) * d;
+        } else if (span_self) {
+            int w0 = kind == 0 ? 0 : hq * d, wn = kind == 0 ? hq * d : hkv * d;
+            const TI* whole = qkv + (size_t)t * ld + w0;
+            // (the numbers are added in the order of the kernel that forms the factors for many tokens, so that a
+            // token's factor does not depend on how many tokens its step has: span_self = 2 is that kernel's order
+            // for rows in 16-byte pieces, a lane taking four neighbours at a time)
+            float s2 = 0.f;
+            if (span_self == 2) {
+                for (int c = lane * 4; c < wn; c += WAVE * 4) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float val = Elem<TI>::load(whole + c + e) + (bias ? bias[w0 + c + e] : 0.f);
+                        s2 = fmaf(val, val, s2);
+                    }
+                }
+            } else {
+                for (int c = lane; c < wn; c += WAVE) {
+                    float val = Elem<TI>::load(whole + c) + (bias ? bias[w0 + c] : 0.f);
+                    s2 = fmaf(val, val, s2);
+                }
+            }
+            inv = 1.0f / sqrtf(wave_sum(s2) / (float)wn + eps);
             gain += (size_t)(kind == 0 ? r : r - hq) * d;
         } else {
             inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
@@ -586,8 +610,10 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, int pairing, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
     const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
-    long long split_stride, const float* bias, int dv, float qt_coef, int qt_every, const float* span_inv,
+    long long split_stride, const float* bias, int dv, float qt_coef, int qt_every, const float* span_inv, int span_self,
     hipStream_t stream) {
+    // span_self: the norm spans a token's whole q row and whole k row as with span_inv, and the kernel forms the
+    // factors itself (a step of few tokens)
     // span_inv (may be null): [T, 2] factors of a norm over a token's whole q row and whole k row (qk_span_stats);
     // q_gain and k_gain then have hq * d and hkv * d numbers.
     // bias (may be null): [ld] numbers added to the projection's sums; dv (0: d): value head size.
@@ -609,9 +635,13 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
                   "qk_norm_rope_append: cache arguments missing");
     ROCML_REQUIRE(q_out || write_kv, "qk_norm_rope_append: nothing to write");
-    ROCML_REQUIRE(!span_inv || (n_splits == 1 && q_gain && k_gain),
+    ROCML_REQUIRE(!(span_inv && span_self), "qk_norm_rope_append: the whole-row norm's factors are given or formed here, not both");
+    ROCML_REQUIRE(!(span_inv || span_self) || (n_splits == 1 && q_gain && k_gain),
                   "qk_norm_rope_append: a norm over the whole projection needs a complete projection and both gains");
     if (n_tokens == 0) return 0;
+    if (span_self)      // the order of additions of qk_span_stats for these rows (see there)
+        span_self = (in_dtype == ROCML_F32 && ld % 4 == 0 && (hq * d) % 4 == 0 && (hkv * d) % 4 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                     (!bias || (uintptr_t)bias % 16 == 0)) ? 2 : 1;
     // prompts: the values go through the transposing tile kernel, the row kernel does q and k
     bool v_tiled = write_kv && n_splits == 1 && n_tokens >= VT_TOKENS;
     // (without q_out the q rows are left to the caller: the prefill attention that reads the
@@ -625,7 +655,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     // (and the pairs are (e, e + d/2): neighbours as pairs go through LDS)
     bool local_pair = per_lane >= 2 && (rot == 0 || (rot == d && pairing == 0)) && d == per_lane * WAVE && dv == d;
     // many rows, none of them values: several rows per wave
-    bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
+    bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv) && !span_self;
     constexpr int MANY = 4;
     int grid = many_rows ? ceil_div(rows, QK_WAVES * MANY) : ceil_div(rows, QK_WAVES);
     size_t lds = local_pair ? 0 : (size_t)QK_WAVES * d * sizeof(float);
@@ -633,7 +663,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv, qt_coef, qt_every, span_inv)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv, qt_coef, qt_every, span_inv, span_self)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \

@@ -558,7 +558,7 @@ __device__ __forceinline__ float rc_logsigmoid(float z) { return fminf(z, 0.f) -
 // operands are asked for as 16-byte pieces, all at once, while the chunk before it is worked on, and reach LDS when
 // that is done.  U tokens are worked on at a time: their operands are all read from LDS first and their sums across
 // lanes run side by side; the gates' recurrence (m, and the two factors of every token) runs ahead of them in
-// every thread.  A token past the chunk's end has keys of zero, a forget gate of one and an input gate of zero
+// every thread; the quotients are formed for the whole chunk afterwards, by all threads at once.  A token past the chunk's end has keys of zero, a forget gate of one and an input gate of zero
 // (log gates 0 and -infinity): it leaves S, n and m as they are, bit for bit.
 template <int NI, bool VEC>
 __global__ void __launch_bounds__(RC_BLOCK)
@@ -576,6 +576,7 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
     float* vs = qs + TC * NP;                  // [TC][SC_PT]
     float* os = vs + TC * SC_PT;               // [TC][SC_PT]
     float* gs = os + TC * SC_PT;               // [TC][2]: log input gate, log forget gate
+    float* dn = gs + 2 * TC;                   // [TC][2]: n . q and m after the token, for the quotient
     int tile = blockIdx.x, p0 = tile * SC_PT, head = blockIdx.y, b = blockIdx.z;
     int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
     int first = cu_seqlens[b], n_tok = cu_seqlens[b + 1] - first;
@@ -659,16 +660,17 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
         }
         for (int t0 = 0; t0 < nt; t0 += U) {
             float2 xv[U];
-            float kv[U][NI], qv[U][NI], fa[U], fb[U], em[U];
+            float kv[U][NI], qv[U][NI], fa[U], fb[U], mt[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 int tt = t0 + u;
                 float2 g = *(const float2*)(gs + 2 * tt);
-                float m_new = fmaxf(g.y + m, g.x);
-                fa[u] = expf(g.y + m - m_new);
-                fb[u] = expf(g.x - m_new);
-                m = m_new;
-                em[u] = expf(-m);
+                // m' = max(f + m, i); of the two factors e^(f + m - m') and e^(i - m') one is e^0 and the other e^(-|i - (f + m)|)
+                float fm = g.y + m, d = g.x - fm, e = expf(-fabsf(d));
+                fa[u] = d > 0.f ? e : 1.f;
+                fb[u] = d > 0.f ? 1.f : e;
+                m = fmaxf(fm, g.x);
+                mt[u] = m;
                 xv[u] = *(const float2*)(vs + tt * SC_PT + pl * SC_PP);
                 const float* kt = ks + tt * NP + r * NI;
                 const float* qt = qs + tt * NP + r * NI;
@@ -710,15 +712,18 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
             if (r == 0) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    float den = fmaxf(fabsf(partn[u]), em[u]) + floor_;
-                    *(float2*)(os + (t0 + u) * SC_PT + pl * SC_PP) = make_float2(part0[u] / den, part1[u] / den);
+                    *(float2*)(os + (t0 + u) * SC_PT + pl * SC_PP) = make_float2(part0[u], part1[u]);
+                    if (tid == 0) *(float2*)(dn + 2 * (t0 + u)) = make_float2(partn[u], mt[u]);
                 }
             }
         }
         __syncthreads();
+        // the quotients, all threads at once: S^T q / (max(|n . q|, e^(-m)) + floor)
         for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
             int tt = i / SC_PT, pp = i - tt * SC_PT;
-            if (p0 + pp < dv) out[(size_t)(first + c0 + tt) * n_heads * dv + (size_t)head * dv + p0 + pp] = os[i];
+            float2 nm = *(const float2*)(dn + 2 * tt);
+            float den = fmaxf(fabsf(nm.x), expf(-nm.y)) + floor_;
+            if (p0 + pp < dv) out[(size_t)(first + c0 + tt) * n_heads * dv + (size_t)head * dv + p0 + pp] = os[i] / den;
         }
     }
 #undef ML_PREFETCH
@@ -780,9 +785,9 @@ mlstm_step_kernel(const float* __restrict__ proj, int ld, int q_col0, int k_col0
     }
     float gi = cap * tanhf((row[i_col0 + head] + (i_bias ? i_bias[head] : 0.f)) / cap);
     float gf = rc_logsigmoid(cap * tanhf((row[f_col0 + head] + (f_bias ? f_bias[head] : 0.f)) / cap));
-    float m_new = fmaxf(gf + m, gi);
-    float a = expf(gf + m - m_new), bb = expf(gi - m_new);
-    m = m_new;
+    float fm = gf + m, d = gi - fm, e = expf(-fabsf(d));
+    float a = d > 0.f ? e : 1.f, bb = d > 0.f ? 1.f : e;
+    m = fmaxf(fm, gi);
     float em = expf(-m);
     float bv0 = bb * xv[0], bv1 = bb * xv[1], q0 = 0.f, q1 = 0.f, nq = 0.f;
 #pragma unroll
@@ -852,7 +857,7 @@ ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_c
         return 0;
     }
     int tc = ni <= 8 ? 32 : 16;
-    size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
+    size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 4 * tc) * sizeof(float);
     // whole 16-byte pieces: every row of q, k and v starts on a multiple of 4 numbers and ends on one
     bool vec = ld % 4 == 0 && dk % 4 == 0 && dv % 4 == 0 && q_col0 % 4 == 0 && k_col0 % 4 == 0 && v_col0 % 4 == 0 &&
                ((uintptr_t)proj & 15) == 0;

@@ -32,7 +32,7 @@ _SIGNATURES = {
         "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _P],
         "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _F, _P],
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
-                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _P],
+                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _I, _P],
         "rocml_qk_span_stats": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P],
         "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P],
         "rocml_layernorm": [_P, _P, _I, _I, _P, _P, _F, _P, _I, _P],
@@ -276,7 +276,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
                         n_splits: int = 1, pairing: str = "halves", bias: Optional[torch.Tensor] = None,
-                        v_head_dim: Optional[int] = None, q_temp=None, span_inv: Optional[torch.Tensor] = None) -> None:
+                        v_head_dim: Optional[int] = None, q_temp=None, span_inv: Optional[torch.Tensor] = None,
+                        span_self: bool = False) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
@@ -288,7 +289,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     ``head_dim``).  ``q_temp``: ``(coef, every)``; the query at position ``p`` is multiplied by
     ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm.  ``span_inv``: ``[T, 2]`` 32-bit, the
     factors of a norm over a token's whole q row and whole k row (``qk_span_stats``); the gains then
-    have one number per column of the q and of the k projection."""
+    have one number per column of the q and of the k projection.  ``span_self``: the same norm, its
+    factors formed inside the kernel (for steps of few tokens)."""
     qt_coef, qt_every = (0.0, 0) if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
     if q_temp is not None and qt_every <= 0:
         raise KernelError(f"the period of the query's stretch must be positive, got {qt_every}")
@@ -308,14 +310,17 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         # (rows may be wider than the projection: a product shared with other mixers, whose columns follow)
         if bias.numel() > ld or bias.numel() < n_heads * head_dim + (n_kv_heads * (head_dim + dv) if write_kv else 0):
             raise KernelError(f"the bias has {bias.numel()} values for rows of {ld}")
+    whole = span_inv is not None or span_self
     if span_inv is not None:
         _want(span_inv, torch.float32, "norm factors")
-        if span_inv.shape != (n_tokens, 2) or n_splits > 1 or q_gain is None or k_gain is None:
-            raise KernelError("a norm over the whole projection needs [tokens, 2] factors, a complete projection and both gains")
+        if span_inv.shape != (n_tokens, 2) or span_self:
+            raise KernelError("the factors of a norm over the whole projection are [tokens, 2], or formed by the kernel itself")
+    if whole and (n_splits > 1 or q_gain is None or k_gain is None or not write_kv):
+        raise KernelError("a norm over the whole projection needs a complete projection with its k columns and both gains")
     for g, heads in ((q_gain, n_heads), (k_gain, n_kv_heads)):
         if g is not None:
             _want(g, torch.float32, "head norm gain")
-            if g.numel() != (head_dim if span_inv is None else heads * head_dim):
+            if g.numel() != (heads * head_dim if whole else head_dim):
                 raise KernelError(f"norm gain has {g.numel()} values for {heads} heads of size {head_dim}")
     if cos is not None:
         if cos.shape != (n_tokens, rot_dim // 2) or sin is None or sin.shape != cos.shape:
@@ -341,7 +346,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out if q_out is not None else k_cache), _ptr(block_table), bt_width, _ptr(token_seq),
         _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _ptr(bias), dv, qt_coef, qt_every,
-        _ptr(span_inv), _stream()))
+        _ptr(span_inv), 1 if span_self else 0, _stream()))
 
 
 def qk_span_stats(qkv: torch.Tensor, q_width: int, k_width: int, bias: Optional[torch.Tensor], eps: float,

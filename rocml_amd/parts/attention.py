@@ -31,6 +31,7 @@ from .residual import stream
 class Attention(Mixer):
     adds_only = True
     FUSED_PREFILL_MIN_TOKENS = 1024
+    SPAN_STATS_MIN_TOKENS = 64         # from so many tokens on, a kernel of its own forms the factors of a whole-row norm of q and k
 
     def __init__(self, spec: AttentionSpec, ctx: BuildContext):
         if spec.n_heads % spec.n_kv_heads != 0:
@@ -250,16 +251,19 @@ class Attention(Mixer):
             else:
                 q = ws.get("attn.q", (n, self.q_dim), self.dtype)
                 bias = None if self.b_qkv is None else self.b_qkv[:rows]
-                span_inv = None
+                span_inv, span_self = None, False
                 if self.span == "projection":
                     if not owns_cache:
                         raise ConfigError("a norm over the whole projection needs the layer's own keys")
-                    span_inv = ws.get("attn.span", (n, 2), torch.float32)
-                    ops.qk_span_stats(qkv, self.q_dim, self.kv_dim, bias, eps, span_inv)
+                    if n < self.SPAN_STATS_MIN_TOKENS:      # few tokens: every wave of the next kernel sums its token's row itself
+                        span_self = True
+                    else:
+                        span_inv = ws.get("attn.span", (n, 2), torch.float32)
+                        ops.qk_span_stats(qkv, self.q_dim, self.kv_dim, bias, eps, span_inv)
                 ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                         cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
                                         step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing,
-                                        bias=bias, v_head_dim=self.v_head_dim, q_temp=s.q_temp, span_inv=span_inv)
+                                        bias=bias, v_head_dim=self.v_head_dim, q_temp=s.q_temp, span_inv=span_inv, span_self=span_self)
                 ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                               s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                               cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,

@@ -169,6 +169,42 @@ def test_window_edges_with_a_norm_over_the_whole_projection(d, dv, H, G, dims, d
     _close(one.reshape(H, dv), want[T - 1], tol, "single-token kernel")
 
 
+@pytest.mark.parametrize("d,dv,H,G,dims", [(40, 40, 4, 2, 12), (24, 40, 3, 3, 24), (128, 128, 4, 2, 128), (64, 64, 16, 1, 0), (10, 6, 1, 1, 2)])
+def test_whole_row_norm_formed_inside_the_kernel(d, dv, H, G, dims):
+    """A step of few tokens has no kernel of its own for the norm's factors: queries and the keys in the cache must
+    come out as with it."""
+    from rocml_amd import ops
+    T, eps = 9, 1e-4
+    g = _gen(d * 7 + H)
+    rot = None if dims == 0 else {"base": 10000.0, "dims": dims}
+    q, k, v = torch.randn(T, H, d, generator=g) * 3, torch.randn(T, G, d, generator=g) * 0.2, torch.randn(T, G, dv, generator=g)
+    qb, kb, vb = 0.3 * torch.randn(H * d, generator=g), 0.3 * torch.randn(G * d, generator=g), 0.3 * torch.randn(G * dv, generator=g)
+    qg, kg = 1 + 0.3 * torch.randn(H * d, generator=g), 1 + 0.3 * torch.randn(G * d, generator=g)
+    positions = list(range(60, 60 + T))                     # across a page's border
+    qkv = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], dim=1).float().to(DEV).contiguous()
+    bias = torch.cat([qb, kb, vb]).float().to(DEV)
+    kc = torch.zeros((4, G, PAGE, d), dtype=torch.float32, device=DEV)
+    vc = torch.zeros((4, G, dv, PAGE), dtype=torch.float32, device=DEV)
+    table = torch.tensor([[2, 0, -1, -1]], dtype=torch.int32, device=DEV)
+    q_out = torch.empty((T, H * d), dtype=torch.float32, device=DEV)
+    seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    cos = sin = None
+    if rot is not None:
+        f, mag = plain.rotary_frequencies(rot)
+        cos = torch.empty(T, dims // 2, dtype=torch.float32, device=DEV)
+        sin = torch.empty_like(cos)
+        ops.rope_table(pos, torch.tensor(f, dtype=D64, device=DEV), cos, sin, mag)
+    ops.qk_norm_rope_append(qkv, H, G, d, qg.to(DEV), kg.to(DEV), eps, cos, sin, dims, q_out, kc, vc, table, seq, pos,
+                            write_kv=True, bias=bias, v_head_dim=dv, span_self=True)
+    qn, kn = _plain_qk(q, k, qb, kb, qg, kg, rot, positions, eps)
+    _close(q_out.reshape(T, H, d), qn, 1e-5, "queries")
+    for j, p in enumerate(positions):
+        page = 2 if p < PAGE else 0
+        _close(kc[page, :, p % PAGE], kn[j], 1e-5, f"key at {p}")
+        _close(vc[page, :, :, p % PAGE], (v[j].reshape(-1).double() + vb.double()).reshape(G, dv), 1e-6, f"value at {p}")
+
+
 def test_gate_per_head():
     from rocml_amd import ops
     g = _gen(5)
