@@ -1281,10 +1281,18 @@ ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float 
 // the new x in another type, for the products that read it next.  One block per row.
 template <typename TC, bool LAYER>
 __global__ void __launch_bounds__(EW_BLOCK)
-norm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
-                const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy) {
+norm_add_kernel(float* __restrict__ x, float* __restrict__ y, const float* __restrict__ gain,
+                const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy,
+                const float* __restrict__ partials, int n_splits, long long split_stride, int replace) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     size_t row = (size_t)blockIdx.x * n;
+    if (n_splits > 0) {         // y (or nothing) plus the K pieces in split order, written back: a thread reads back its own
+        for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+            float v = replace ? 0.f : y[row + i];
+            for (int sp = 0; sp < n_splits; ++sp) v += partials[sp * split_stride + row + i];
+            y[row + i] = v;
+        }
+    }
     float mean = 0.f;
     if (LAYER) {
         float s = 0.f;
@@ -1311,7 +1319,8 @@ norm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float*
 template <typename TC, bool LAYER, int VEC>
 __global__ void __launch_bounds__(EW_BLOCK)
 norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
-                    const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy) {
+                    const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy,
+                    const float* __restrict__ partials, int n_splits, long long split_stride, int replace) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     size_t row = (size_t)blockIdx.x * n;
     int nv = n / 4;
@@ -1321,10 +1330,21 @@ norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const fl
     for (int j = 0; j < VEC; ++j) {
         int i = threadIdx.x + j * EW_BLOCK;
         bool ok = i < nv;
-        yv[j] = ok ? ((const float4*)(y + row))[i] : zero4;
+        yv[j] = (ok && !replace) ? ((const float4*)(y + row))[i] : zero4;
         xv[j] = ok ? ((const float4*)(x + row))[i] : zero4;
         gv[j] = ok ? ((const float4*)gain)[i] : zero4;
         bv[j] = (ok && LAYER && bias) ? ((const float4*)bias)[i] : zero4;
+    }
+    // the K pieces of the product that made y, in split order
+    for (int sp = 0; sp < n_splits; ++sp) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            int i = threadIdx.x + j * EW_BLOCK;
+            if (i < nv) {
+                float4 p = ((const float4*)(partials + sp * split_stride + row))[i];
+                yv[j].x += p.x; yv[j].y += p.y; yv[j].z += p.z; yv[j].w += p.w;
+            }
+        }
     }
     float mean = 0.f;
     if (LAYER) {
@@ -1358,13 +1378,14 @@ norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const fl
 }
 
 template <typename TC, bool LAYER>
-static void launch_norm_add(float* x, const float* y, const float* gain, const float* bias, float eps, int n_rows, int n,
-                            TC* copy, hipStream_t stream) {
+static void launch_norm_add(float* x, float* y, const float* gain, const float* bias, float eps, int n_rows, int n,
+                            TC* copy, const float* partials, int n_splits, long long split_stride, int replace, hipStream_t stream) {
     bool vec = n % 4 == 0 && n <= 4 * EW_BLOCK * RN_MAX_VEC && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
-               (uintptr_t)gain % 16 == 0 && (!bias || (uintptr_t)bias % 16 == 0) && (!copy || (uintptr_t)copy % 8 == 0);
+               (uintptr_t)gain % 16 == 0 && (!bias || (uintptr_t)bias % 16 == 0) && (!copy || (uintptr_t)copy % 8 == 0) &&
+               (n_splits == 0 || ((uintptr_t)partials % 16 == 0 && split_stride % 4 == 0));
     int v = ceil_div(n / 4, EW_BLOCK);
-#define NAV(V_) norm_add_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy)
-    if (!vec) norm_add_kernel<TC, LAYER><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy);
+#define NAV(V_) norm_add_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace)
+    if (!vec) norm_add_kernel<TC, LAYER><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace);
     else if (v <= 1) NAV(1);
     else if (v <= 2) NAV(2);
     else if (v <= 4) NAV(4);
@@ -1372,19 +1393,24 @@ static void launch_norm_add(float* x, const float* y, const float* gain, const f
 #undef NAV
 }
 
-ROCML_EXPORT int rocml_norm_add(float* x, const float* y, int n_rows, int n, const float* gain, const float* bias,
-                                float eps, int layer, void* copy, int copy_dtype, hipStream_t stream) {
+ROCML_EXPORT int rocml_norm_add(float* x, float* y, int n_rows, int n, const float* gain, const float* bias,
+                                float eps, int layer, void* copy, int copy_dtype, const float* partials, int n_splits,
+                                long long split_stride, int replace, hipStream_t stream) {
     // layer = 1: layer norm (mean taken off, bias added if given); 0: root-mean-square norm (bias is not read)
+    // partials (may be null): [n_splits][rows][n] K pieces of the product that made y, added to y in split order first;
+    // with replace they are all of y (what y holds is not read; the plain kernel uses y as its buffer)
     ROCML_REQUIRE(n_rows >= 0 && n > 0 && x && y && gain, "norm_add: bad arguments rows=%d n=%d", n_rows, n);
+    ROCML_REQUIRE(n_splits >= 0 && (n_splits == 0 ? !replace : (partials && split_stride >= (long long)n_rows * n)),
+                  "norm_add: %d partial sums with a stride of %lld do not fit", n_splits, split_stride);
     ROCML_REQUIRE(!copy || copy_dtype == ROCML_F32 || copy_dtype == ROCML_BF16, "norm_add: unknown dtype code %d", copy_dtype);
     if (n_rows == 0) return 0;
     bool half = copy && copy_dtype == ROCML_BF16;
     if (layer) {
-        if (half) launch_norm_add<bf16_t, true>(x, y, gain, bias, eps, n_rows, n, (bf16_t*)copy, stream);
-        else launch_norm_add<float, true>(x, y, gain, bias, eps, n_rows, n, (float*)copy, stream);
+        if (half) launch_norm_add<bf16_t, true>(x, y, gain, bias, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, stream);
+        else launch_norm_add<float, true>(x, y, gain, bias, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, stream);
     } else {
-        if (half) launch_norm_add<bf16_t, false>(x, y, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, stream);
-        else launch_norm_add<float, false>(x, y, gain, nullptr, eps, n_rows, n, (float*)copy, stream);
+        if (half) launch_norm_add<bf16_t, false>(x, y, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, stream);
+        else launch_norm_add<float, false>(x, y, gain, nullptr, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, stream);
     }
     ROCML_CHECK_LAUNCH("norm_add");
     return 0;

@@ -60,12 +60,13 @@ class Workspace:
     # its partial sums in the scratch memory; the next kernel that reads the tensor (a norm)
     # adds them itself.  Whoever needs the scratch memory or the tensor before that calls
     # flush_pending, which runs the addition as a kernel of its own.
-    def set_pending(self, target: torch.Tensor, n_splits: int) -> None:
+    def set_pending(self, target: torch.Tensor, n_splits: int, replace: bool = False) -> None:
+        """``replace``: the partial sums are all of ``target``'s new value (what it holds does not count)."""
         self.flush_pending()
-        self._pending = (target, n_splits)
+        self._pending = (target, n_splits, replace)
 
     def _partials(self) -> torch.Tensor:
-        target, n_splits = self._pending
+        target, n_splits = self._pending[:2]
         n = n_splits * target.numel()
         return self._scratch[:n * 4].view(torch.float32).view(n_splits, target.shape[0], target.shape[1])
 
@@ -74,20 +75,32 @@ class Workspace:
         now adds itself; None if there are none."""
         if self._pending is None:
             return None
-        if self._pending[0].data_ptr() != target.data_ptr():
+        if self._pending[0].data_ptr() != target.data_ptr() or self._pending[2]:
             self.flush_pending()
             return None
         partials = self._partials()
         self._pending = None
         return partials
 
+    def take_pending_or_whole(self, target: torch.Tensor):
+        """``(partial sums, replace)`` waiting for ``target``: with ``replace`` they are all of its value, without it
+        they are to be added to what it holds; None if there are none.  The caller now adds them itself."""
+        if self._pending is None:
+            return None
+        if self._pending[0].data_ptr() != target.data_ptr():
+            self.flush_pending()
+            return None
+        partials, replace = self._partials(), self._pending[2]
+        self._pending = None
+        return partials, replace
+
     def flush_pending(self) -> None:
         if self._pending is not None:
             from .. import ops
             partials = self._partials()
-            target = self._pending[0]
+            target, replace = self._pending[0], self._pending[2]
             self._pending = None
-            ops.splitk_reduce(partials, target, accumulate=True)
+            ops.splitk_reduce(partials, target, accumulate=not replace)
 
     def drop_pending(self) -> None:
         self._pending = None

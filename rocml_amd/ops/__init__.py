@@ -34,7 +34,7 @@ _SIGNATURES = {
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
                                       _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _I, _P],
         "rocml_qk_span_stats": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P],
-        "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P],
+        "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P, _I, _LL, _I, _P],
         "rocml_layernorm": [_P, _P, _I, _I, _P, _P, _F, _P, _I, _P],
         "rocml_token_side_gate": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
@@ -364,10 +364,21 @@ def qk_span_stats(qkv: torch.Tensor, q_width: int, k_width: int, bias: Optional[
 
 
 def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
-             layer: bool, copy: Optional[torch.Tensor] = None) -> None:
+             layer: bool, copy: Optional[torch.Tensor] = None, partials: Optional[torch.Tensor] = None,
+             replace: bool = False) -> None:
     """``x += f(y)`` row by row in 32-bit: ``f`` a layer norm ``(y - mean) / sqrt(var + eps) * gain + bias``
-    (``layer``) or ``y / sqrt(mean(y^2) + eps) * gain``.  ``copy`` gets the new ``x`` in its own type."""
-    _dev(x, y, gain, bias, copy)
+    (``layer``) or ``y / sqrt(mean(y^2) + eps) * gain``.  ``copy`` gets the new ``x`` in its own type.
+    ``partials`` (``[splits, rows, n]`` 32-bit): the K pieces of the product that made ``y``, added to ``y`` in
+    split order first, or with ``replace`` all of ``y`` (what ``y`` holds is not read)."""
+    _dev(x, y, gain, bias, copy, partials)
+    n_splits = split_stride = 0
+    if partials is not None:
+        _want(partials, torch.float32, "partial sums")
+        if partials.dim() != 3 or tuple(partials.shape[1:]) != tuple(x.shape):
+            raise KernelError("norm_add: partial sums must be [splits, rows, n]")
+        n_splits, split_stride = partials.shape[0], x.numel()
+    elif replace:
+        raise KernelError("norm_add: nothing to replace the sublayer's output with")
     for t, what in ((x, "residual stream"), (y, "sublayer output"), (gain, "norm gain")):
         _want(t, torch.float32, what)
     if x.dim() != 2 or y.shape != x.shape or gain.numel() != x.shape[1] or (copy is not None and copy.shape != x.shape) \
@@ -375,7 +386,7 @@ def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optiona
         raise KernelError("norm_add: shapes do not fit")
     _check("elementwise", library("elementwise").rocml_norm_add(
         _ptr(x), _ptr(y), x.shape[0], x.shape[1], _ptr(gain), _ptr(bias), float(eps), 1 if layer else 0, _ptr(copy),
-        _code(copy) if copy is not None else 0, _stream()))
+        _code(copy) if copy is not None else 0, _ptr(partials), n_splits, split_stride, 1 if replace else 0, _stream()))
 
 
 def layernorm(x: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float, out: torch.Tensor,

@@ -262,7 +262,11 @@ class SublayerNormBlock(Part):
         copy = None
         if self.dtype != torch.float32:
             copy = step.workspace.get("block.stream_copy", tuple(x.shape), self.dtype)
-        ops.norm_add(x, y, norm.gain, getattr(norm, "bias", None), norm.eps, layer=bool(getattr(norm, "centred", False)), copy=copy)
+        # (a product cut along K may have left its pieces for this kernel to add: they are all of y then)
+        pending = step.workspace.take_pending_or_whole(y)
+        partials, replace = pending if pending is not None else (None, False)
+        ops.norm_add(x, y, norm.gain, getattr(norm, "bias", None), norm.eps, layer=bool(getattr(norm, "centred", False)), copy=copy,
+                     partials=partials, replace=replace)
         if copy is not None:
             step.memo[_COPY_KEY] = (x.data_ptr(), copy)
 
@@ -274,21 +278,19 @@ class SublayerNormBlock(Part):
         try:
             xb = self._operand(step, x)
             y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
-            rs.overwrite = True
+            rs.overwrite = rs.defer_overwrite = True
             self.mixer.forward(step, xb, y, cache, owns_cache)
-            ws.flush_pending()
             self._norm_add(step, x, y, self.children["mixer_norm"])
             for part, norm in ((self.ffn, "ffn_norm"), (self.side, "side_norm")):
                 if part is None:
                     continue
                 xb = self._operand(step, x)
                 y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
-                rs.overwrite = True
+                rs.overwrite = rs.defer_overwrite = True
                 part.forward(step, xb, y)
-                ws.flush_pending()
                 self._norm_add(step, x, y, self.children[norm])
         finally:
-            rs.overwrite = False
+            rs.overwrite = rs.defer_overwrite = False
 
 
 register_block("sublayer_norm", SublayerNormBlock)

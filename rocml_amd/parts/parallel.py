@@ -83,7 +83,8 @@ class ParallelMixer(Mixer):
         ``weight * sum_b rms(outputs[b]) * gains[b]``; the outputs are 32-bit ``[tokens, hidden]``."""
         ws = step.workspace
         rs = stream(step)
-        before = rs.overwrite
+        before, before_defer = rs.overwrite, rs.defer_overwrite
+        rs.defer_overwrite = False        # the branches' outputs are read by a kernel that takes whole sums
         views = cache.parts if cache is not None else (None,) * len(self.children)
         outs: List[torch.Tensor] = []
         proj = None
@@ -99,7 +100,7 @@ class ParallelMixer(Mixer):
                 child.forward(step, xn, y, views[i], owns_cache)
             ws.flush_pending()
             outs.append(y)
-        rs.overwrite = before
+        rs.overwrite, rs.defer_overwrite = before, before_defer
         return outs, [self.gains[name] for name in self.children], float(self.spec.weight)
 
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:

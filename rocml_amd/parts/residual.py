@@ -37,6 +37,8 @@ class ResidualStream:
         # set around a part's forward by a block whose sublayers do not add to the stream: the part's
         # target is a buffer of the block's, and the part's last product writes it instead of adding to it
         self.overwrite = False
+        # with ``overwrite``: the block's next kernel can add a product's K pieces itself (``take_pending_or_whole``)
+        self.defer_overwrite = False
         self._prescaled = None
 
     def add_product(self, a: torch.Tensor, w: torch.Tensor, target: torch.Tensor) -> None:
@@ -47,7 +49,9 @@ class ResidualStream:
         self._prescaled = None
         if self.overwrite:
             ws.flush_pending()
-            ops.gemm(a, w, target, accumulate=False, workspace=ws.scratch())
+            splits = ops.gemm(a, w, target, accumulate=False, workspace=ws.scratch(), defer=self.defer_overwrite)
+            if splits:
+                ws.set_pending(target, splits, replace=True)
             return
         if hint is not None and target.dtype == torch.float32 and hint.width == target.shape[1] \
                 and ops.gemm_residual_prescale_pays(a, w):

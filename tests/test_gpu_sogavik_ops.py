@@ -53,6 +53,28 @@ def test_layer_norm_and_sublayer_norm_added_to_the_stream(n):
                 _close(copy, want, 1e-2 if copy_type == torch.bfloat16 else 1e-5, "copy")
 
 
+@pytest.mark.parametrize("n", [36, 211, 1024, 8200])
+def test_sublayer_norm_adds_the_pieces_of_a_product(n):
+    """The kernel is handed a product's K pieces instead of its sum: on top of what the buffer holds, or as all of it."""
+    from rocml_amd import ops
+    g = _gen(n + 1)
+    rows, eps = 5, 1e-5
+    x, y = torch.randn(rows, n, generator=g), torch.randn(rows, n, generator=g)
+    parts = torch.randn(3, rows, n, generator=g) * 2
+    w, b = 1 + 0.3 * torch.randn(n, generator=g), 0.5 * torch.randn(n, generator=g)
+    for replace in (False, True):
+        total = parts.double().sum(0) + (0 if replace else y.double())
+        for layer, want in ((True, x.double() + plain.layer_norm(total, w.double(), b.double(), eps)),
+                            (False, x.double() + plain.rms(total, eps) * w.double())):
+            xs = x.clone().to(DEV)
+            ys = (y.clone() if not replace else torch.full((rows, n), float("nan"))).to(DEV)
+            copy = torch.empty(rows, n, dtype=torch.bfloat16, device=DEV)
+            ops.norm_add(xs, ys, w.to(DEV), b.to(DEV) if layer else None, eps, layer=layer, copy=copy, partials=parts.to(DEV),
+                         replace=replace)
+            _close(xs, want, 1e-5, f"stream, layer={layer}, replace={replace}")
+            _close(copy, want, 1e-2, "copy")
+
+
 def test_rotation_table_with_a_magnitude():
     from rocml_amd import ops
     rot = {"base": 5000.0, "dims": 12, "scaling": {"factor": 3.0, "original": 64, "fast": 8.0, "slow": 2.0}}
