@@ -119,20 +119,20 @@ CATALOG += [
 def sogavik_config(vocab, width, heads, kv_heads, dim, window, mem_heads, mem_dim, experts, expert_ff, top, side_dim, n_layers,
                    parallel_every=4, max_positions=40960):
     """A Sogavik configuration: windowed attention with a gate per head in most layers (its rotation's
-    frequencies stretched fourfold beyond 4,096 positions), and in every ``parallel_every``-th layer (the third
+    frequencies stretched eightfold beyond 4,096 positions), and in every ``parallel_every``-th layer (the third
     among them) a windowed attention of a quarter of the window beside a matrix memory; routed experts in every
     layer, and ``side_dim`` columns of the side table for each."""
     def attention(w, stretched):
         rot = {"base": 1000000.0, "dims": dim}
         if stretched:
-            rot["scaling"] = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+            rot["scaling"] = {"factor": 8.0, "original": 4096, "fast": 24.0, "slow": 2.0}
         return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": w}, "rot": rot}
     mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}
     layers = []
     for i in range(n_layers):
         if i % parallel_every == min(2, parallel_every - 1):
             mixer = {"left": attention(max(window // 4, 1), False),
-                     "right": {"heads": mem_heads, "dim": mem_dim, "vdim": mem_dim, "gate_cap": 15.0}}
+                     "right": {"heads": mem_heads, "dim": mem_dim, "vdim": mem_dim, "gate_cap": 10.0}}
             layers.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
         else:
             layers.append({"type": "attention", "mixer": attention(window, True), "mlp": mlp})

@@ -63,8 +63,8 @@ CFG_A = config(211, 72, [
 # are multiples of 8, windows of 64, 65 and 130 (a page, a page and one, two pages and two), the parallel layers
 # first and last.  Its attention scales are twice 1/sqrt(dim): it is the model that bfloat16 runs are judged on.
 CFG_B = config(300, 128, [
-    parallel_layer(attention(4, 1, 64, 64, 0.25, 65, (10000.0, 64)), memory(2, 64, 64, 15.0), moe(8, 64, 3)),
-    attention_layer(attention(2, 2, 128, 128, 0.18, 130, (1000000.0, 64), (4.0, 128, 16.0, 1.0)), moe(16, 32, 4)),
+    parallel_layer(attention(4, 1, 64, 64, 0.25, 65, (10000.0, 64)), memory(2, 64, 64, 12.0), moe(8, 64, 3)),
+    attention_layer(attention(2, 2, 128, 128, 0.18, 130, (200000.0, 64), (5.0, 128, 16.0, 1.0)), moe(16, 32, 4)),
     attention_layer(attention(8, 4, 32, 32, 0.35, 64, (10000.0, 32), (8.0, 64, 8.0, 2.0)), None),
     parallel_layer(attention(4, 2, 64, 64, 0.3, 200, (500.0, 16)), memory(4, 128, 32, 30.0), moe(4, 96, 2)),
 ], side_dim=8)

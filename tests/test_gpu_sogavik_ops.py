@@ -321,7 +321,7 @@ def test_matrix_memory_gates_at_their_limits(forget, take):
     of nearly zero drops it at once; input gates at the cap on either side; the running maximum starts at zero, so
     small input gates are not scaled up."""
     g = _gen(int(forget + 2 * take) + 100)
-    H, dk, dv, T, cap = 2, 24, 40, 300, 15.0
+    H, dk, dv, T, cap = 2, 24, 40, 300, 20.0
     cols = (0, H * dk, 2 * H * dk, 2 * H * dk + H * dv, 2 * H * dk + H * dv + H)
     proj = torch.randn(T, cols[4] + H, generator=g)
     # (queries and keys of one sign: n . q is then a sum without cancellation, and what is compared is the

@@ -84,10 +84,10 @@ def test_config_round_trip_and_refusals():
             arch.read_config(bad)
 
 
-@pytest.mark.parametrize("rot", [{"base": 1000000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 128, "fast": 16.0, "slow": 1.0}},
+@pytest.mark.parametrize("rot", [{"base": 200000.0, "dims": 64, "scaling": {"factor": 5.0, "original": 128, "fast": 16.0, "slow": 1.0}},
                                  {"base": 5000.0, "dims": 12, "scaling": {"factor": 3.0, "original": 64, "fast": 8.0, "slow": 2.0}},
                                  {"base": 100.0, "dims": 20, "scaling": {"factor": 1.0, "original": 16, "fast": 2.0, "slow": 1.0}},
-                                 {"base": 10000.0, "dims": 2, "scaling": {"factor": 16.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+                                 {"base": 10000.0, "dims": 2, "scaling": {"factor": 16.0, "original": 4096, "fast": 24.0, "slow": 1.5}},
                                  {"base": 300.0, "dims": 4}])
 def test_stretched_frequencies(rot):
     """The rotation part's frequencies and magnitude against the plain function; with a stretch, some frequencies
@@ -104,7 +104,7 @@ def test_stretched_frequencies(rot):
     if rot["dims"] == 64:
         bare = [rot["base"] ** (-2.0 * i / 64) for i in range(32)]
         ratio = [a / b for a, b in zip(f, bare)]
-        assert ratio[0] == 1.0 and abs(ratio[-1] - 0.25) < 1e-12 and any(0.26 < r < 0.99 for r in ratio)
+        assert ratio[0] == 1.0 and abs(ratio[-1] - 0.2) < 1e-12 and any(0.21 < r < 0.99 for r in ratio)
 
 
 def test_cache_lines_of_the_matrix_memory():
