@@ -1,6 +1,7 @@
 """Sogavik on the CPU: configuration reading, tensor names, the parts a layer is made of, the stretched
 rotation's frequencies, and the cache's bookkeeping for the matrix memory's state."""
 import copy
+import json
 
 import pytest
 import torch
@@ -136,3 +137,20 @@ def test_cache_lines_of_the_matrix_memory():
         "a slot that is used again starts from a zero state and a running maximum of zero"
     cache.free_sequence(b)
     cache.check()
+
+
+def test_random_model_folder_has_the_checkpoint_names(tmp_path):
+    """``init`` for a catalog entry of this design writes config.json and every tensor under its checkpoint name."""
+    from safetensors import safe_open
+    from rocml_amd.config.catalog import resolve
+    from rocml_amd.weights import write_model_dir
+    cfg = resolve("sogavik-tiny").entry.config
+    path = write_model_dir(str(tmp_path / "m"), cfg, 5, dtype=torch.bfloat16, norm_jitter=True)
+    arch, spec = _spec(cfg)
+    model = DecoderModel(spec, torch.float32, device="meta")
+    names = arch.checkpoint_names(spec)
+    with safe_open(f"{path}/model.safetensors", "pt") as f:
+        found = {k: tuple(f.get_slice(k).get_shape()) for k in f.keys()}
+    assert found == {names[k]: tuple(p.shape) for k, p in model.param_specs().items()}
+    assert "side.embed" in found and found["side.embed"] == (cfg["vocab"], len(cfg["layers"]) * cfg["token_side"]["dim"])
+    assert architecture_of(json.load(open(f"{path}/config.json"))).name == "Sogavik"
