@@ -2,7 +2,7 @@
 """Decode and prefill speed of the Qwen3 shapes with random bfloat16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-8b|qwen3-14b|qwen3-32b]
-    python bench.py --design dokulix|felovik|sogavik [--design-size 2b|8b] [--layers N]
+    python bench.py --design dokulix|felovik|sogavik [--design-size 2b|8b|14b] [--layers N]
 
 The default run is the Qwen3-8B shape.  A step is one decode step of a batch of 8 sequences,
 each with a 2,048-token random prompt in the cache (context length 4,096): the engine's step
@@ -59,6 +59,8 @@ DESIGN_SIZES = {
                window=1024, chunk=1024, vocab=32768),
     "8b": dict(width=4096, ff=12288, heads=32, kv_heads=8, dim=128, q_rank=1536, kv_rank=512, rot_dim=64,
                window=1024, chunk=1024, vocab=32768),
+    "14b": dict(width=5120, ff=17408, heads=40, kv_heads=8, dim=128, q_rank=1536, kv_rank=512, rot_dim=64,
+                window=1024, chunk=1024, vocab=32768),
 }
 
 
