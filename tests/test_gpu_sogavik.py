@@ -25,7 +25,10 @@ TOL = {"float32": 3e-4}
 # experts and reaches every later position: the 32-bit runs pin every position, the bfloat16 runs pin the bulk of
 # them against the plain implementation and against each other.
 BF16_MOST = {"A": (0.5, 5e-2), "B": (0.5, 4e-2), "C": (0.5, 1e-1), "D": (0.5, 5e-2)}
-BF16_SAME = {"A": (0.9, 4e-2), "B": (0.9, 6e-2), "C": (0.9, 4e-2), "D": (0.9, 4e-2)}
+# (one flipped choice of experts late in a sequence of 64 puts an eighth of its positions off in one of the two runs: B,
+# whose head sizes take the matrix-core attention with its differently rounding prompt and single-token kernels, is
+# held to four positions in five)
+BF16_SAME = {"A": (0.9, 4e-2), "B": (0.8, 6e-2), "C": (0.9, 4e-2), "D": (0.9, 4e-2)}
 LENGTHS = {"A": [1, 2, 21, 66, 150, 211], "B": [3, 64, 65, 131, 262], "C": [1, 8, 30, 77], "D": [5, 40, 129]}
 
 
