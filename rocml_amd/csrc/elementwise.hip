@@ -1393,6 +1393,120 @@ static void launch_norm_add(float* x, float* y, const float* gain, const float* 
 #undef NAV
 }
 
+// The same with the sublayer's output still in branches: y = c * sum_b y_b / sqrt(mean(y_b^2) + eps_b) * gain_b (one or two
+// mixers that ran side by side, each normed over the width with a gain of its own) is formed in registers, in the
+// order of operations of sum_norm, and normed and added as above.  Rows of up to 4096 values that are multiples of 4.
+template <typename TC, bool LAYER, int VEC>
+__global__ void __launch_bounds__(EW_BLOCK)
+norm_add_branches_vec_kernel(float* __restrict__ x, const float* __restrict__ y0, const float* __restrict__ y1,
+                             const float* __restrict__ g0, const float* __restrict__ g1, float c, float eps_b,
+                             const float* __restrict__ gain, const float* __restrict__ bias, float eps, int n,
+                             TC* __restrict__ copy) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    size_t row = (size_t)blockIdx.x * n;
+    int nv = n / 4;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 av[VEC], bv2[VEC], ga[VEC], gb[VEC], xv[VEC], gv[VEC], bv[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        bool ok = i < nv;
+        av[j] = ok ? ((const float4*)(y0 + row))[i] : zero4;
+        ga[j] = ok ? ((const float4*)g0)[i] : zero4;
+        bv2[j] = (ok && y1) ? ((const float4*)(y1 + row))[i] : zero4;
+        gb[j] = (ok && y1) ? ((const float4*)g1)[i] : zero4;
+        xv[j] = ok ? ((const float4*)(x + row))[i] : zero4;
+        gv[j] = ok ? ((const float4*)gain)[i] : zero4;
+        bv[j] = (ok && LAYER && bias) ? ((const float4*)bias)[i] : zero4;
+    }
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        s0 = fmaf(av[j].x, av[j].x, s0); s0 = fmaf(av[j].y, av[j].y, s0); s0 = fmaf(av[j].z, av[j].z, s0); s0 = fmaf(av[j].w, av[j].w, s0);
+        s1 = fmaf(bv2[j].x, bv2[j].x, s1); s1 = fmaf(bv2[j].y, bv2[j].y, s1); s1 = fmaf(bv2[j].z, bv2[j].z, s1); s1 = fmaf(bv2[j].w, bv2[j].w, s1);
+    }
+    float inv0 = 1.0f / sqrtf(block_sum(s0, scratch) / (float)n + eps_b);
+    float inv1 = y1 ? 1.0f / sqrtf(block_sum(s1, scratch) / (float)n + eps_b) : 0.f;
+    float4 yv[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        float4 sum;
+        sum.x = av[j].x * inv0 * ga[j].x; sum.y = av[j].y * inv0 * ga[j].y; sum.z = av[j].z * inv0 * ga[j].z; sum.w = av[j].w * inv0 * ga[j].w;
+        if (y1) {
+            sum.x += bv2[j].x * inv1 * gb[j].x; sum.y += bv2[j].y * inv1 * gb[j].y;
+            sum.z += bv2[j].z * inv1 * gb[j].z; sum.w += bv2[j].w * inv1 * gb[j].w;
+        }
+        yv[j] = make_float4(c * sum.x, c * sum.y, c * sum.z, c * sum.w);
+    }
+    float mean = 0.f;
+    if (LAYER) {
+        float sm = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) sm += (yv[j].x + yv[j].y) + (yv[j].z + yv[j].w);
+        mean = block_sum(sm, scratch) / (float)n;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        if (threadIdx.x + j * EW_BLOCK < nv) {
+            yv[j].x -= mean; yv[j].y -= mean; yv[j].z -= mean; yv[j].w -= mean;
+        }
+        ss = fmaf(yv[j].x, yv[j].x, ss); ss = fmaf(yv[j].y, yv[j].y, ss);
+        ss = fmaf(yv[j].z, yv[j].z, ss); ss = fmaf(yv[j].w, yv[j].w, ss);
+    }
+    float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        if (i >= nv) continue;
+        float4 v;
+        v.x = xv[j].x + (yv[j].x * inv * gv[j].x + bv[j].x);
+        v.y = xv[j].y + (yv[j].y * inv * gv[j].y + bv[j].y);
+        v.z = xv[j].z + (yv[j].z * inv * gv[j].z + bv[j].z);
+        v.w = xv[j].w + (yv[j].w * inv * gv[j].w + bv[j].w);
+        ((float4*)(x + row))[i] = v;
+        if (copy) store4(copy + row + 4 * (size_t)i, v.x, v.y, v.z, v.w);
+    }
+}
+
+constexpr int NAB_MAX_N = 4 * EW_BLOCK * 4;      // the widest row the kernel above keeps in registers
+
+ROCML_EXPORT int rocml_norm_add_branches_fits(int n) { return n > 0 && n % 4 == 0 && n <= NAB_MAX_N; }
+
+template <typename TC, bool LAYER>
+static void launch_norm_add_branches(float* x, const float* y0, const float* y1, const float* g0, const float* g1, float c,
+                                     float eps_b, const float* gain, const float* bias, float eps, int n_rows, int n, TC* copy,
+                                     hipStream_t stream) {
+    int v = ceil_div(n / 4, EW_BLOCK);
+#define NAB(V_) norm_add_branches_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y0, y1, g0, g1, c, eps_b, gain, bias, eps, n, copy)
+    if (v <= 1) NAB(1);
+    else if (v <= 2) NAB(2);
+    else NAB(4);
+#undef NAB
+}
+
+ROCML_EXPORT int rocml_norm_add_branches(float* x, const float* y0, const float* y1, const float* g0, const float* g1,
+                                         float c, float eps_b, int n_rows, int n, const float* gain, const float* bias,
+                                         float eps, int layer, void* copy, int copy_dtype, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && x && y0 && g0 && gain && (!y1 || g1), "norm_add_branches: missing arguments");
+    ROCML_REQUIRE(rocml_norm_add_branches_fits(n), "norm_add_branches: rows of %d values (a multiple of 4, at most %d)", n, NAB_MAX_N);
+    ROCML_REQUIRE(!copy || copy_dtype == ROCML_F32 || copy_dtype == ROCML_BF16, "norm_add_branches: unknown dtype code %d", copy_dtype);
+    const void* ptrs[] = {x, y0, y1, g0, g1, gain, bias};
+    for (const void* q : ptrs) ROCML_REQUIRE((uintptr_t)q % 16 == 0, "norm_add_branches: operands must start on 16 bytes");
+    ROCML_REQUIRE(!copy || (uintptr_t)copy % 8 == 0, "norm_add_branches: the copy must start on 8 bytes");
+    if (n_rows == 0) return 0;
+    bool half = copy && copy_dtype == ROCML_BF16;
+    if (layer) {
+        if (half) launch_norm_add_branches<bf16_t, true>(x, y0, y1, g0, g1, c, eps_b, gain, bias, eps, n_rows, n, (bf16_t*)copy, stream);
+        else launch_norm_add_branches<float, true>(x, y0, y1, g0, g1, c, eps_b, gain, bias, eps, n_rows, n, (float*)copy, stream);
+    } else {
+        if (half) launch_norm_add_branches<bf16_t, false>(x, y0, y1, g0, g1, c, eps_b, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, stream);
+        else launch_norm_add_branches<float, false>(x, y0, y1, g0, g1, c, eps_b, gain, nullptr, eps, n_rows, n, (float*)copy, stream);
+    }
+    ROCML_CHECK_LAUNCH("norm_add_branches");
+    return 0;
+}
+
 ROCML_EXPORT int rocml_norm_add(float* x, float* y, int n_rows, int n, const float* gain, const float* bias,
                                 float eps, int layer, void* copy, int copy_dtype, const float* partials, int n_splits,
                                 long long split_stride, int replace, hipStream_t stream) {

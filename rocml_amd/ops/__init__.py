@@ -35,6 +35,8 @@ _SIGNATURES = {
                                       _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _I, _P],
         "rocml_qk_span_stats": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P],
         "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P, _I, _LL, _I, _P],
+        "rocml_norm_add_branches": [_P, _P, _P, _P, _P, _F, _F, _I, _I, _P, _P, _F, _I, _P, _I, _P],
+        "rocml_norm_add_branches_fits": [_I],
         "rocml_layernorm": [_P, _P, _I, _I, _P, _P, _F, _P, _I, _P],
         "rocml_token_side_gate": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
@@ -387,6 +389,32 @@ def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optiona
     _check("elementwise", library("elementwise").rocml_norm_add(
         _ptr(x), _ptr(y), x.shape[0], x.shape[1], _ptr(gain), _ptr(bias), float(eps), 1 if layer else 0, _ptr(copy),
         _code(copy) if copy is not None else 0, _ptr(partials), n_splits, split_stride, 1 if replace else 0, _stream()))
+
+
+def norm_add_branches_fits(n: int, n_branches: int) -> bool:
+    """Whether ``norm_add_branches`` takes rows of ``n`` values in ``n_branches`` branches."""
+    return 1 <= n_branches <= 2 and bool(library("elementwise").rocml_norm_add_branches_fits(int(n)))
+
+
+def norm_add_branches(x: torch.Tensor, branches: Sequence[torch.Tensor], branch_gains: Sequence[torch.Tensor], weight: float,
+                      branch_eps: float, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float, layer: bool,
+                      copy: Optional[torch.Tensor] = None) -> None:
+    """``x += f(weight * sum_b rms(y_b) * gain_b)`` row by row in 32-bit for one or two branches ``y_b``, each divided by
+    its own root mean square (``branch_eps`` inside the root) first; ``f`` as in ``norm_add``."""
+    _dev(x, gain, bias, copy, *branches, *branch_gains)
+    if not norm_add_branches_fits(x.shape[1], len(branches)) or len(branch_gains) != len(branches):
+        raise KernelError(f"norm_add_branches takes one or two branches of rows it can keep in registers, got {len(branches)} of {x.shape[1]}")
+    for t in (x, gain, *branches, *branch_gains):
+        _want(t, torch.float32, "stream, branches and gains")
+    n = x.shape[1]
+    if any(y.shape != x.shape for y in branches) or any(g.numel() != n for g in branch_gains) or gain.numel() != n \
+            or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != n)) or (copy is not None and copy.shape != x.shape):
+        raise KernelError("norm_add_branches: shapes do not fit")
+    y1 = branches[1] if len(branches) > 1 else None
+    g1 = branch_gains[1] if len(branches) > 1 else None
+    _check("elementwise", library("elementwise").rocml_norm_add_branches(
+        _ptr(x), _ptr(branches[0]), _ptr(y1), _ptr(branch_gains[0]), _ptr(g1), float(weight), float(branch_eps), x.shape[0], n,
+        _ptr(gain), _ptr(bias), float(eps), 1 if layer else 0, _ptr(copy), _code(copy) if copy is not None else 0, _stream()))
 
 
 def layernorm(x: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float, out: torch.Tensor,

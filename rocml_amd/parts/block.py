@@ -270,6 +270,25 @@ class SublayerNormBlock(Part):
         if copy is not None:
             step.memo[_COPY_KEY] = (x.data_ptr(), copy)
 
+    def _branches_norm_add(self, step, x, xb, cache, owns_cache: bool) -> bool:
+        """A mixer that is a sum of normed branches hands them over as they are: one kernel norms the branches, sums
+        them, norms the sum and adds it to the stream.  False: the mixer is of another kind, or its rows do not fit
+        that kernel (the mixer then forms its sum itself)."""
+        if not hasattr(self.mixer, "branches") or not ops.norm_add_branches_fits(self.hidden, len(self.mixer.children)):
+            return False
+        outs, gains, weight = self.mixer.branches(step, xb, cache, owns_cache)
+        if any(g is None for g in gains):
+            raise ConfigError("the branches of a parallel mixer come with a gain each")
+        norm = self.children["mixer_norm"]
+        copy = None
+        if self.dtype != torch.float32:
+            copy = step.workspace.get("block.stream_copy", tuple(x.shape), self.dtype)
+        ops.norm_add_branches(x, outs, gains, weight, self.mixer.spec.eps, norm.gain, getattr(norm, "bias", None), norm.eps,
+                              layer=bool(getattr(norm, "centred", False)), copy=copy)
+        if copy is not None:
+            step.memo[_COPY_KEY] = (x.data_ptr(), copy)
+        return True
+
     def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
         ws = step.workspace
         rs = stream(step)
@@ -279,8 +298,9 @@ class SublayerNormBlock(Part):
             xb = self._operand(step, x)
             y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
             rs.overwrite = rs.defer_overwrite = True
-            self.mixer.forward(step, xb, y, cache, owns_cache)
-            self._norm_add(step, x, y, self.children["mixer_norm"])
+            if not self._branches_norm_add(step, x, xb, cache, owns_cache):
+                self.mixer.forward(step, xb, y, cache, owns_cache)
+                self._norm_add(step, x, y, self.children["mixer_norm"])
             for part, norm in ((self.ffn, "ffn_norm"), (self.side, "side_norm")):
                 if part is None:
                     continue

@@ -127,6 +127,8 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
         qkv.shape[0] * (q_width + k_width) * qkv.element_size() + _nbytes(out), 2 * qkv.shape[0] * (q_width + k_width))),
     "norm_add": ("sublayer norm and residual sum", lambda x, y, gain, bias, eps, **kw: (
         2 * _nbytes(x) + _nbytes(kw.get("copy"), kw.get("partials")) + (0 if kw.get("replace") else _nbytes(y)), 8 * x.numel())),
+    "norm_add_branches": ("branch norms, sublayer norm and residual sum", lambda x, branches, gains, weight, beps, gain, bias, eps, layer, **kw: (
+        2 * _nbytes(x) + _nbytes(*branches) + _nbytes(kw.get("copy")), 8 * x.numel() * (1 + len(branches)))),
     "layernorm": ("layer norm", lambda x, gain, bias, eps, out, rows=None: (out.numel() * 4 + _nbytes(out), 8 * out.numel())),
     "token_side_gate": ("token-side gate", lambda g, table, ids, col0, out, *a, **kw: (
         _nbytes(g, out, ids) + out.numel() * table.element_size(), 10 * out.numel())),

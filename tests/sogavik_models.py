@@ -86,7 +86,14 @@ CFG_D = config(97, 48, [
     attention_layer(attention(3, 1, 16, 8, 0.9, 12, (1000.0, 16)), moe(4, 24, 1)),
 ], side_dim=None)
 
-CONFIGS = {"A": (CFG_A, 31), "B": (CFG_B, 32), "C": (CFG_C, 33), "D": (CFG_D, 34)}
+# E: a width that is no multiple of 4 (no kernel takes its rows as 16-byte pieces, and the pair of mixers forms its sum in
+# a kernel of its own), both kinds of layer.
+CFG_E = config(90, 70, [
+    parallel_layer(attention(2, 1, 12, 10, 0.8, 6, (100.0, 6)), memory(2, 5, 7, 3.0), moe(3, 10, 2)),
+    attention_layer(attention(2, 2, 10, 14, 0.9, 20, (100.0, 10), (2.0, 8, 4.0, 1.0)), moe(2, 18, 1)),
+], side_dim=3)
+
+CONFIGS = {"A": (CFG_A, 31), "B": (CFG_B, 32), "C": (CFG_C, 33), "D": (CFG_D, 34), "E": (CFG_E, 35)}
 
 
 def _attention_shapes(p: str, m: Dict, w: int, gate: bool) -> Dict[str, tuple]:

@@ -75,6 +75,32 @@ def test_sublayer_norm_adds_the_pieces_of_a_product(n):
             _close(copy, want, 1e-2, "copy")
 
 
+@pytest.mark.parametrize("n", [36, 72, 1024, 4096])
+@pytest.mark.parametrize("n_branches", [1, 2])
+def test_branch_norms_sublayer_norm_and_sum_in_one_kernel(n, n_branches):
+    """Two mixers' outputs of very different size, each normed over the width with its own gain, half their sum, its
+    norm, the residual sum and the copy."""
+    from rocml_amd import ops
+    g = _gen(n + n_branches)
+    rows, eps_b, eps = 6, 1e-4, 1e-3
+    x = torch.randn(rows, n, generator=g)
+    ys = [torch.randn(rows, n, generator=g) * s + 0.5 for s in (20.0, 0.05)][:n_branches]
+    gs = [1 + 0.3 * torch.randn(n, generator=g) for _ in ys]
+    w, b = 1 + 0.3 * torch.randn(n, generator=g), 0.5 * torch.randn(n, generator=g)
+    assert ops.norm_add_branches_fits(n, n_branches) and not ops.norm_add_branches_fits(70, 2) and not ops.norm_add_branches_fits(8192, 2)
+    total = 0.5 * sum(plain.rms(y.double(), eps_b) * gg.double() for y, gg in zip(ys, gs))
+    for layer, want in ((True, x.double() + plain.layer_norm(total, w.double(), b.double(), eps)),
+                        (False, x.double() + plain.rms(total, eps) * w.double())):
+        for copy_type in (None, torch.bfloat16, torch.float32):
+            xs = x.clone().to(DEV)
+            copy = None if copy_type is None else torch.empty(rows, n, dtype=copy_type, device=DEV)
+            ops.norm_add_branches(xs, [y.to(DEV) for y in ys], [gg.to(DEV) for gg in gs], 0.5, eps_b, w.to(DEV),
+                                  b.to(DEV) if layer else None, eps, layer=layer, copy=copy)
+            _close(xs, want, 1e-5, f"stream, layer={layer}")
+            if copy is not None:
+                _close(copy, want, 1e-2 if copy_type == torch.bfloat16 else 1e-5, "copy")
+
+
 def test_rotation_table_with_a_magnitude():
     from rocml_amd import ops
     rot = {"base": 5000.0, "dims": 12, "scaling": {"factor": 3.0, "original": 64, "fast": 8.0, "slow": 2.0}}

@@ -20,7 +20,7 @@ def _spec(cfg):
     return arch, arch.to_spec(arch.read_config(cfg))
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_tensor_names_and_shapes(name):
     cfg, _ = sm.CONFIGS[name]
     arch, spec = _spec(cfg)
