@@ -29,6 +29,9 @@ class Architecture:
     checkpoint_names: Callable[[ModelSpec], Dict[str, str]]
     # names of tensors a checkpoint may hold although the model does not read them
     unused_tensors: Callable[[ModelSpec], Any] = lambda spec: ()
+    # (configuration, {tensor name: shape}) -> configuration: fills in sizes that config.json leaves to the
+    # checkpoint's tensor shapes; None if the configuration says everything
+    refine_config: Any = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -125,6 +128,14 @@ def _register_builtin() -> None:
         to_spec=lambda cfg: cfg.to_model_spec(),
         checkpoint_names=sogavik.checkpoint_names,
         unused_tensors=sogavik.unused_tensors))
+    from . import roravik
+    register_architecture(Architecture(
+        name=roravik.ARCHITECTURE,
+        read_config=roravik.RoravikConfig.from_dict,
+        to_spec=lambda cfg: cfg.to_model_spec(),
+        checkpoint_names=roravik.checkpoint_names,
+        unused_tensors=roravik.unused_tensors,
+        refine_config=lambda cfg, shapes: cfg.with_shapes(shapes)))
 
 
 _register_builtin()

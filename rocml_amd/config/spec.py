@@ -84,7 +84,12 @@ class AttentionSpec:
     ``o_bias``: whether the output projection has a bias when it is not what ``bias`` says (None: as
     ``bias``).  ``qk_norm_span``: ``"head"``, every head of q and of k is normed by itself with a gain
     of the head's size, or ``"projection"``, a token's whole q row (all heads side by side) is
-    normed at once with a gain of that size, and its k row likewise."""
+    normed at once with a gain of that size, and its k row likewise.  ``sink_learned`` (with ``sink``):
+    the extra term is ``exp(sink_h)`` with a learned number per query head instead of ``exp(0)``.
+    ``softcap``: the scaled score ``s`` becomes ``softcap * tanh(s / softcap)`` before the mask.
+    ``conv``: q, k and v pass a causal convolution of so many taps per channel (no bias, no
+    activation) right after their projection; the last ``conv - 1`` projected rows of a sequence
+    are part of its state."""
     hidden: int
     n_heads: int
     n_kv_heads: int
@@ -104,6 +109,9 @@ class AttentionSpec:
     gate_per_head: bool = False
     o_bias: Optional[bool] = None
     qk_norm_span: str = "head"
+    sink_learned: bool = False
+    softcap: Optional[float] = None
+    conv: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -155,7 +163,12 @@ class RoutedExpertsSpec:
     the ``keep`` best groups can be chosen.  The chosen experts' scores, divided by their sum plus
     ``sum_eps``, weight their outputs.  ``weighting`` ``"softmax_chosen"`` instead: the experts with
     the largest logits are chosen and the weights are the softmax over the chosen logits alone (no
-    groups).  ``router_bias``: a bias vector is added to the router's logits."""
+    groups).  ``router_bias``: a bias vector is added to the router's logits.  ``weighting`` ``"sigmoid"``:
+    an expert's score is ``sigmoid(logit)`` by itself.  ``correction``: a learned number per expert is added to the
+    scores for the choice (of groups and of experts) only; the weights use the scores without it.
+    ``group_score`` ``"top2_sum"``: a group's score is the sum of its two largest (corrected) scores instead of
+    its largest.  ``shared_intermediate``: one more expert of that size runs for every token and is added, with
+    ``shared_gate`` times ``sigmoid(W_sg h)`` (one number per token)."""
     hidden: int
     n_experts: int
     top: int
@@ -166,6 +179,10 @@ class RoutedExpertsSpec:
     kind: str = "routed_experts"
     weighting: str = "softmax_all"
     router_bias: bool = False
+    correction: bool = False
+    group_score: str = "max"
+    shared_intermediate: Optional[int] = None
+    shared_gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -211,6 +228,40 @@ class MatrixMemorySpec:
 
 
 @dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with one fixed decay per head and neither softmax nor denominator:
+    ``q = W_q h``, ``k = W_k h`` (rotated as ``position`` says, k then times ``head_dim^(-1/2)``),
+    ``v = W_v h``; per head ``S <- decay_h S + k v^T`` and ``o = S^T q`` with the new ``S``.  Every head's
+    output is divided by its root mean square, the heads side by side are multiplied by
+    ``silu(W_g h)`` and projected back.  The state (``head_dim x v_head_dim`` per head) is 32-bit."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_head_dim: int
+    decay: Tuple[float, ...]
+    eps: float
+    position: Optional[RopeSpec] = None
+    kind: str = "retention"
+
+
+@dataclass(frozen=True)
+class TimeMixSpec:
+    """A recurrence whose decay depends on the token, per head and key channel (the time mixing of
+    RWKV-6).  With ``h'`` the previous token's input (zeros before the first), each of r, k, v, g, w
+    reads its own mix ``h + (h' - h) mu``; ``r``, ``k``, ``v`` are ``n_heads x head_dim`` wide;
+    ``w = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0))`` with an inner width of ``decay_rank``; per head
+    ``o = (S + diag(u) k v^T)^T r``, then ``S <- diag(w) S + k v^T``.  Every head's output is divided by
+    its root mean square, the heads side by side are multiplied by a gain and by ``silu(W_g mix_g)``
+    and projected back.  The state and the previous token's input live per sequence."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    decay_rank: int
+    eps: float
+    kind: str = "time_mix"
+
+
+@dataclass(frozen=True)
 class TokenSideSpec:
     """A per-token input that depends on the token's id: with ``e`` the columns ``column0 ..
     column0 + dim - 1`` of the token's row of the model's table ``table``, the result is
@@ -236,12 +287,16 @@ class ParallelMixerSpec:
     """A set of mixers that all run on one input.  The result is
     ``weight * sum_b norm_b(out_b)``: each branch's output is normed over the model width with a
     gain of its own.  ``branches`` are ``(name, mixer spec)`` pairs; a branch's parameters and
-    its output norm carry its name."""
+    its output norm carry its name.  ``normed`` false: the branches' outputs are taken as they
+    are.  ``branch_weights``: one factor per branch, ``sum_b branch_weights[b] * f_b(out_b)`` (then
+    ``weight`` is not used)."""
     hidden: int
     branches: Tuple[Tuple[str, Any], ...]
     weight: float
     eps: float
     kind: str = "parallel"
+    normed: bool = True
+    branch_weights: Optional[Tuple[float, ...]] = None
 
 
 @dataclass(frozen=True)
@@ -267,12 +322,14 @@ class TokenPositionTableSpec:
 @dataclass(frozen=True)
 class NormLinearHeadSpec:
     """The model's output: a norm of the wanted rows of the residual stream, then their
-    product with a ``[vocab, hidden]`` matrix; ``tied``: that matrix is the input's table."""
+    product with a ``[vocab, hidden]`` matrix; ``tied``: that matrix is the input's table.
+    ``softcap``: the logits ``z`` become ``softcap * tanh(z / softcap)``."""
     vocab: int
     hidden: int
     norm: NormSpec
     tied: bool
     kind: str = "norm_linear"
+    softcap: Optional[float] = None
 
 
 @dataclass(frozen=True)
@@ -286,7 +343,9 @@ class BlockSpec:
     sublayers read the stream itself and the norms come after the sums.  ``sublayer_norm`` is
     ``x += norm(mixer(x)); x += norm(ffn(x))``: the sublayers read the stream itself and a norm
     is applied to a sublayer's output alone.  ``side`` (with ``side_norm``): one more sublayer
-    that runs last in the same way (only in ``sublayer_norm``)."""
+    that runs last in the same way (only in ``sublayer_norm``).  ``sandwich_norm`` is
+    ``x += mixer_out_norm(mixer(mixer_norm(x))); x += ffn_out_norm(ffn(ffn_norm(x)))``: a norm before
+    and one after every sublayer."""
     mixer: Any
     ffn: Any
     mixer_norm: Any
@@ -295,6 +354,8 @@ class BlockSpec:
     residual_scale: float = 1.0
     side: Any = None
     side_norm: Optional[Any] = None
+    mixer_out_norm: Optional[Any] = None
+    ffn_out_norm: Optional[Any] = None
 
 
 @dataclass(frozen=True)
@@ -304,10 +365,13 @@ class ScheduleEntry:
     line of its own).  ``reads_cache_of`` names an earlier entry of the schedule
     whose cache line this execution reads instead of writing its own.  ``offset_row``: row of
     the model's table of pass offsets (``ModelSpec.pass_offsets`` rows of ``hidden`` values) that
-    is added to the residual stream of every token right before this execution."""
+    is added to the residual stream of every token right before this execution.  ``add_embedding``:
+    the embedding's output for the step's tokens (the stream as it was before the first entry) is
+    added to the stream right before this execution."""
     layer: int
     reads_cache_of: Optional[int] = None
     offset_row: Optional[int] = None
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -328,6 +392,7 @@ class ModelSpec:
     head: Any = None
     pass_offsets: int = 0                   # rows of the table that schedule entries add to the stream
     tables: Tuple[Any, ...] = ()            # matrices that parts of several layers read (``TableSpec``)
+    logit_softcap: Optional[float] = None   # the default head's soft cap on the logits
 
     def embedding_spec(self) -> Any:
         return self.embedding if self.embedding is not None else \
@@ -335,7 +400,7 @@ class ModelSpec:
 
     def head_spec(self) -> Any:
         return self.head if self.head is not None else \
-            NormLinearHeadSpec(self.vocab, self.hidden, self.final_norm, self.tie_lm_head)
+            NormLinearHeadSpec(self.vocab, self.hidden, self.final_norm, self.tie_lm_head, softcap=self.logit_softcap)
 
     def validate(self) -> None:
         from ..errors import ConfigError

@@ -195,8 +195,10 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
                                  const int* cu_seqlens, int n_seqs, int max_new, const int* q_counts,
                                  int max_len, int n_splits, void* workspace, long long workspace_bytes,
                                  int dv, int v_in_k, int chunk, const float* slopes, int sink,
-                                 hipStream_t stream) {
-    // dv (0: the key head's size), v_in_k, chunk, slopes and sink: see AttnExtra in attention_generic.h.
+                                 const float* sinks, float softcap, hipStream_t stream) {
+    // dv (0: the key head's size), v_in_k, chunk, slopes, sink, sinks and softcap: see AttnExtra in attention_generic.h.
+    ROCML_REQUIRE(!sinks || sink, "attention: learned sinks need the sink switched on");
+    ROCML_REQUIRE(softcap >= 0.f, "attention: negative soft cap %g", (double)softcap);
     if (dv <= 0) dv = d;
     ROCML_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "attention: a layer has a window or blocks of positions, not both");
     ROCML_REQUIRE(!v_in_k || dv <= d, "attention: values taken from the key rows need dv <= d (dv=%d d=%d)", dv, d);
@@ -204,7 +206,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(dv <= AG_BLOCK * AG_MAX_D_PER_THREAD, "attention: value head size %d exceeds %d", dv,
                   AG_BLOCK * AG_MAX_D_PER_THREAD);
     bool plain_features = dv == d && !v_in_k;          // what the matrix-core kernels need
-    bool has_extra = chunk > 0 || slopes || sink;
+    bool has_extra = chunk > 0 || slopes || sink || softcap > 0.f;
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0 && page_size > 0 && bt_width > 0,
                   "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d width=%d", n_tokens, hq, hkv,
                   d, page_size, bt_width);
@@ -262,7 +264,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
         AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
                    bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, (int)total_q_tiles, max_len, hq, hkv,
                    scale, window, workspace, workspace_bytes, n_splits, nullptr};
-        a.extra = MaskExtra{chunk, slopes, sink};
+        a.extra = MaskExtra{chunk, slopes, sink, sinks, softcap};
         a.has_extra = has_extra;
         int rc = decode ? BY_HEAD_DIM(launch_decode_plain, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
         if (rc) return rc;
@@ -271,7 +273,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     }
     dim3 grid(n_tokens, hq);
     size_t lds = (size_t)(d + AG_BLOCK) * sizeof(float);
-    AttnExtra ex{dv, v_in_k, chunk, slopes, sink};
+    AttnExtra ex{dv, v_in_k, chunk, slopes, sink, sinks, softcap};
     if (dtype == ROCML_F32)
         attn_generic_kernel<float><<<grid, AG_BLOCK, lds, stream>>>(
             (const float*)q, (float*)out, (const float*)kcache, (const float*)vcache, block_table,

@@ -16,7 +16,9 @@
 //    up to itself (lo = pos - pos % chunk) instead of a window;
 //  * slopes[h]: slope * (pos - j) is taken off the score of key j;
 //  * sink: one more term exp(0) in the denominator, with no value: the running maximum starts at 0
-//    and the running sum at 1.
+//    and the running sum at 1;
+//  * sinks[h]: with sink, the term is exp(sinks[h]) instead: the running maximum starts there;
+//  * softcap: the scaled score s becomes softcap * tanh(s / softcap), before the mask and the slope.
 #pragma once
 #include "common.h"
 
@@ -51,6 +53,8 @@ struct AttnExtra {
     int chunk;              // 0: none
     const float* slopes;    // [Hq] or null
     int sink;
+    const float* sinks;     // [Hq] or null
+    float softcap;          // 0: none
 };
 
 __device__ __forceinline__ int attn_first_key(int pos, int window, int chunk) {
@@ -78,7 +82,7 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
     const T* qrow = q + ((size_t)t * hq + h) * d;
     for (int e = tid; e < d; e += AG_BLOCK) qs[e] = Elem<T>::load(qrow + e);
     __syncthreads();
-    float m = ex.sink ? 0.f : -INFINITY, l = ex.sink ? 1.f : 0.f;
+    float m = ex.sink ? (ex.sinks ? ex.sinks[h] : 0.f) : -INFINITY, l = ex.sink ? 1.f : 0.f;
     float acc[AG_MAX_D_PER_THREAD] = {};
     for (int c0 = lo; c0 <= pos; c0 += AG_BLOCK) {
         int j = c0 + tid;
@@ -88,7 +92,9 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
             const T* krow = kcache + (((size_t)page * hkv + kvh) * page_size + j % page_size) * d;
             float dot = 0.f;
             for (int e = 0; e < d; ++e) dot = fmaf(qs[e], Elem<T>::load(krow + e), dot);
-            s = dot * scale - slope * (float)(pos - j);
+            s = dot * scale;
+            if (ex.softcap > 0.f) s = ex.softcap * tanhf(s / ex.softcap);
+            s -= slope * (float)(pos - j);
         }
         float m_new = fmaxf(m, ag_block_max(s, red));
         float corr = expf(m - m_new);            // first chunk: exp(-inf) = 0

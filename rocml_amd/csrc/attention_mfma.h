@@ -73,8 +73,15 @@ struct MaskExtra {
     int chunk;              // > 0: a query sees the keys of its own block of `chunk` positions (counted from 0) up to itself
     const float* slopes;    // [Hq] or null: slope * (query position - key position) is taken off a score
     int sink;               // one more term exp(0) in the softmax's denominator, with no value
+    const float* sinks;     // [Hq] or null: with `sink`, the term is exp(sinks[head]) instead
+    float softcap;          // > 0: the scaled score s becomes softcap * tanh(s / softcap) before the mask
 };
 constexpr float AM_LOG2E = 1.4426950408889634f;
+// tanh by one exponential and one reciprocal (both hardware approximations; the kernels here round to bfloat16 anyway)
+__device__ __forceinline__ float am_tanh(float x) {
+    float e = __builtin_amdgcn_exp2f(fminf(x * (2.0f * AM_LOG2E), 64.f));
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
 
 template <int D, bool FUSED, int AHEAD, int WAVES, bool EXTRA = false>
 __global__ void __launch_bounds__(64 * WAVES)
@@ -111,6 +118,11 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             from_start = false;
         }
         if (mx.slopes) slope_l2 = mx.slopes[kvh * group + min(col, group - 1)] * AM_LOG2E;
+    }
+    // the soft cap in the units of the scores as they are exponentiated (powers of two)
+    float cap_in = 0.f, cap_out = 0.f;
+    if constexpr (EXTRA) {
+        if (mx.softcap > 0.f) { cap_in = 1.0f / (mx.softcap * AM_LOG2E); cap_out = mx.softcap * AM_LOG2E; }
     }
     int first_page = lo / AM_PAGE;
     int n_pages = (len + AM_PAGE - 1) / AM_PAGE - first_page;
@@ -278,7 +290,10 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     float m = -INFINITY, l = 0.f;
     if constexpr (EXTRA) {
         // the sink is one key of score 0 and value 0: it enters once, in the first wave of the first split
-        if (mx.sink && split == 0 && wave == 0) { m = 0.f; l = 1.f; }
+        if (mx.sink && split == 0 && wave == 0) {
+            m = mx.sinks ? mx.sinks[kvh * group + min(col, group - 1)] * AM_LOG2E : 0.f;
+            l = 1.f;
+        }
     }
     f32x4_t o[DT];
 #pragma unroll
@@ -305,7 +320,11 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 int key = key0 + g * 8 + u * 4 + i;
-                float v = (key >= from && key < to) ? s[u][i] * scale_log2e : -INFINITY;
+                float v = s[u][i] * scale_log2e;
+                if constexpr (EXTRA) {
+                    if (cap_out != 0.f) v = am_tanh(v * cap_in) * cap_out;
+                }
+                v = (key >= from && key < to) ? v : -INFINITY;
                 if constexpr (EXTRA) v -= slope_l2 * (float)(len - 1 - key);
                 s[u][i] = v;
                 mx = fmaxf(mx, v);
@@ -531,6 +550,14 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     if constexpr (EXTRA) {
         if (mx.slopes) kslope = mx.slopes[h] * AM_LOG2E / scale_log2e;
     }
+    // the soft cap, into and out of the units of the raw dot products
+    float cap_in = 0.f, cap_out = 0.f;
+    if constexpr (EXTRA) {
+        if (mx.softcap > 0.f) {
+            cap_in = scale_log2e / (AM_LOG2E * mx.softcap);
+            cap_out = mx.softcap * AM_LOG2E / scale_log2e;
+        }
+    }
     int wave_last_key = pos0 + w_hi;
 
     // Q^T operand: column = query row, 8 values of D per lane and step.
@@ -597,7 +624,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     }
     float m = -INFINITY, l = 0.f;
     if constexpr (EXTRA) {
-        if (mx.sink) { m = 0.f; l = 1.f; }            // one key of score 0 and value 0 in every row
+        if (mx.sink) { m = mx.sinks ? mx.sinks[h] * AM_LOG2E : 0.f; l = 1.f; }   // one key of score 0 (or sinks[h]) and value 0 in every row
     }
     f32x16_t o[DT];
 #pragma unroll
@@ -675,6 +702,12 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             int key0 = page_key0 + half * 32;
             f32x16_t& s = sc[half];
             bool need_mask = !wave_full || key0 + 31 > wave_min_pos || key0 < wave_max_lo;   // wave-uniform
+            if constexpr (EXTRA) {
+                if (cap_out != 0.f) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) s[e] = am_tanh(s[e] * cap_in) * cap_out;
+                }
+            }
             if (need_mask) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {

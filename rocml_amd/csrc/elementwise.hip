@@ -1621,3 +1621,68 @@ ROCML_EXPORT int rocml_convert(const float* x, void* out, int out_dtype, long lo
     ROCML_CHECK_LAUNCH("convert");
     return 0;
 }
+
+// ---- soft cap ----------------------------------------------------------------------------
+// x <- cap * tanh(x / cap), in place, 32-bit (a model's logits).
+__global__ void softcap_kernel(float* __restrict__ x, float cap, float inv_cap, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx < total) x[idx] = cap * tanhf(x[idx] * inv_cap);
+}
+
+ROCML_EXPORT int rocml_softcap(float* x, float cap, long long total, hipStream_t stream) {
+    ROCML_REQUIRE(total >= 0 && x && cap > 0.f, "softcap: bad arguments (cap %g)", (double)cap);
+    if (total == 0) return 0;
+    softcap_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(x, cap, 1.0f / cap, total);
+    ROCML_CHECK_LAUNCH("softcap");
+    return 0;
+}
+
+// ---- weighted sum of up to four matrices ------------------------------------------------------
+// out <- alpha * out + sum_b w[b] * y[b], all 32-bit and of one shape (alpha 0: out is only written).
+struct WeightedSumArgs {
+    const float* y[4];
+    float w[4];
+};
+
+__global__ void weighted_sum_kernel(float* __restrict__ out, WeightedSumArgs a, int n_branches, float alpha, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    float acc = alpha != 0.f ? alpha * out[idx] : 0.f;
+    for (int b = 0; b < n_branches; ++b) acc = fmaf(a.w[b], a.y[b][idx], acc);
+    out[idx] = acc;
+}
+
+ROCML_EXPORT int rocml_weighted_sum(float* out, const float* const* ys, const float* weights, int n_branches, float alpha,
+                                    long long total, hipStream_t stream) {
+    ROCML_REQUIRE(total >= 0 && out && ys && weights && n_branches >= 1 && n_branches <= 4, "weighted_sum: bad arguments (%d branches)",
+                  n_branches);
+    if (total == 0) return 0;
+    WeightedSumArgs a{};
+    for (int b = 0; b < n_branches; ++b) {
+        ROCML_REQUIRE(ys[b], "weighted_sum: branch %d is missing", b);
+        a.y[b] = ys[b];
+        a.w[b] = weights[b];
+    }
+    weighted_sum_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(out, a, n_branches, alpha, total);
+    ROCML_CHECK_LAUNCH("weighted_sum");
+    return 0;
+}
+
+// ---- a matrix added row by row under a gate --------------------------------------------------
+// x[t, :] += sigmoid(g[t * ldg]) * y[t, :], 32-bit: a part that every token uses, weighed by one number per token.
+__global__ void row_gate_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ g, int ldg, int n,
+                                    long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / n;
+    x[idx] = fmaf(1.0f / (1.0f + expf(-g[(size_t)t * ldg])), y[idx], x[idx]);
+}
+
+ROCML_EXPORT int rocml_row_gate_add(float* x, const float* y, const float* g, int ldg, int n_rows, int n, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0 && ldg >= 1 && x && y && g, "row_gate_add: bad arguments rows=%d n=%d", n_rows, n);
+    long long total = (long long)n_rows * n;
+    if (total == 0) return 0;
+    row_gate_add_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(x, y, g, ldg, n, total);
+    ROCML_CHECK_LAUNCH("row_gate_add");
+    return 0;
+}

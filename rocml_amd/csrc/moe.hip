@@ -29,16 +29,22 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
     }
 }
 
+// sigmoid != 0: s = sigmoid(logit) by itself instead of the softmax.  correction (may be null): one number per
+// expert that is added to s for the choice (of groups and of experts) only; the weights use s without it, so a
+// choice score may be negative and "cannot be chosen" is minus infinity.  group_top2: a group's score is the sum
+// of its two largest choice scores (of its one score in groups of one expert).
 __global__ void __launch_bounds__(RT_BLOCK)
 moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, int top, int group_count, int group_keep,
-                 float sum_eps, int* __restrict__ chosen, float* __restrict__ weight, const float* __restrict__ bias) {
+                 float sum_eps, int* __restrict__ chosen, float* __restrict__ weight, const float* __restrict__ bias,
+                 int sigmoid, const float* __restrict__ correction, int group_top2, int ld) {
+    // ld: numbers between the starts of two tokens' logits (the logits may be the leading columns of a wider matrix)
     // bias (may be null): one number per expert, added to the logits first
     extern __shared__ float rt_smem[];          // [waves][n_experts]
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     int t = blockIdx.x * (RT_BLOCK / WAVE) + wave;
     bool live = t < n_tokens;
     float* mine = rt_smem + (size_t)wave * n_experts;
-    const float* z = logits + (size_t)(live ? t : 0) * n_experts;
+    const float* z = logits + (size_t)(live ? t : 0) * ld;
     float s[RT_MAX_PER_LANE];
     float m = -INFINITY;
 #pragma unroll
@@ -47,80 +53,93 @@ moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, 
         s[j] = e < n_experts ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
         m = fmaxf(m, s[j]);
     }
-    m = wave_max(m);
-    float sum = 0.f;
+    if (sigmoid) {
 #pragma unroll
-    for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
-        int e = lane + j * WAVE;
-        s[j] = e < n_experts ? expf(s[j] - m) : 0.f;
-        sum += s[j];
-    }
-    sum = wave_sum(sum);
+        for (int j = 0; j < RT_MAX_PER_LANE; ++j) s[j] = lane + j * WAVE < n_experts ? 1.0f / (1.0f + expf(-s[j])) : 0.f;
+    } else {
+        m = wave_max(m);
+        float sum = 0.f;
 #pragma unroll
-    for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
-        int e = lane + j * WAVE;
-        s[j] = s[j] / sum;
-        if (e < n_experts) mine[e] = s[j];
+        for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
+            int e = lane + j * WAVE;
+            s[j] = e < n_experts ? expf(s[j] - m) : 0.f;
+            sum += s[j];
+        }
+        sum = wave_sum(sum);
+#pragma unroll
+        for (int j = 0; j < RT_MAX_PER_LANE; ++j) s[j] = s[j] / sum;
     }
-    // candidates: -1 marks an expert that cannot be chosen (any more)
+    // candidates: the choice scores; minus infinity marks an expert that cannot be chosen (any more)
     float cand[RT_MAX_PER_LANE];
 #pragma unroll
-    for (int j = 0; j < RT_MAX_PER_LANE; ++j) cand[j] = lane + j * WAVE < n_experts ? s[j] : -1.f;
+    for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
+        int e = lane + j * WAVE;
+        cand[j] = e < n_experts ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+        if (e < n_experts) mine[e] = cand[j];
+    }
     if (group_count > 0) {
         __syncthreads();
         int per = n_experts / group_count;
         // group scores, one or more groups per lane
         float gs[RT_MAX_PER_LANE];
+        bool kept[RT_MAX_PER_LANE];
 #pragma unroll
         for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
             int g = lane + j * WAVE;
-            gs[j] = -1.f;
+            gs[j] = -INFINITY;
+            kept[j] = false;
             if (g < group_count) {
-                float best = mine[g * per];
-                for (int i = 1; i < per; ++i) best = fmaxf(best, mine[g * per + i]);
-                gs[j] = best;
+                float best = mine[g * per], second = -INFINITY;
+                for (int i = 1; i < per; ++i) {
+                    float c = mine[g * per + i];
+                    if (c > best) { second = best; best = c; }
+                    else if (c > second) second = c;
+                }
+                gs[j] = group_top2 && per > 1 ? best + second : best;
             }
         }
-        // the kept groups, best first; a kept group's score is set to -2 so that it marks itself
+        // the kept groups, best first
         for (int k = 0; k < group_keep; ++k) {
-            float bv = -1.f;
+            float bv = -INFINITY;
             int bi = 0x7fffffff;
 #pragma unroll
             for (int j = 0; j < RT_MAX_PER_LANE; ++j)
-                if (gs[j] > bv) { bv = gs[j]; bi = lane + j * WAVE; }
+                if (lane + j * WAVE < group_count && !kept[j] && (gs[j] > bv || bi == 0x7fffffff)) { bv = gs[j]; bi = lane + j * WAVE; }
             wave_argmax(bv, bi);
 #pragma unroll
             for (int j = 0; j < RT_MAX_PER_LANE; ++j)
-                if (lane + j * WAVE == bi) gs[j] = -2.f;
+                if (lane + j * WAVE == bi) kept[j] = true;
         }
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
             int g = lane + j * WAVE;
-            if (g < group_count) mine[g] = gs[j] == -2.f ? 1.f : 0.f;      // (scores are in registers by now)
+            if (g < group_count) mine[g] = kept[j] ? 1.f : 0.f;      // (scores are in registers by now)
         }
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < RT_MAX_PER_LANE; ++j) {
             int e = lane + j * WAVE;
-            if (e < n_experts && mine[e / per] == 0.f) cand[j] = -1.f;
+            if (e < n_experts && mine[e / per] == 0.f) cand[j] = -INFINITY;
         }
     }
     float total = 0.f;
     float mine_w = 0.f;
     int mine_e = 0;
     for (int k = 0; k < top; ++k) {
-        float bv = -1.f;
+        float bv = -INFINITY;
         int bi = 0x7fffffff;
 #pragma unroll
         for (int j = 0; j < RT_MAX_PER_LANE; ++j)
             if (cand[j] > bv) { bv = cand[j]; bi = lane + j * WAVE; }
         wave_argmax(bv, bi);
+        float sv = 0.f;
 #pragma unroll
         for (int j = 0; j < RT_MAX_PER_LANE; ++j)
-            if (lane + j * WAVE == bi) cand[j] = -1.f;
-        total += bv;
-        if (lane == k) { mine_w = bv; mine_e = bi; }
+            if (lane + j * WAVE == bi) { cand[j] = -INFINITY; sv = s[j]; }
+        sv = wave_sum(sv);            // the chosen expert's score, from the lane that holds it
+        total += sv;
+        if (lane == k) { mine_w = sv; mine_e = bi; }
     }
     if (live && lane < top) {
         chosen[(size_t)t * top + lane] = mine_e;
@@ -129,7 +148,9 @@ moe_route_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, 
 }
 
 ROCML_EXPORT int rocml_moe_route(const float* logits, int n_tokens, int n_experts, int top, int group_count, int group_keep,
-                                 float sum_eps, int* chosen, float* weight, const float* bias, hipStream_t stream) {
+                                 float sum_eps, int* chosen, float* weight, const float* bias, int sigmoid,
+                                 const float* correction, int group_top2, int ld, hipStream_t stream) {
+    ROCML_REQUIRE(ld >= n_experts, "moe_route: rows of %d numbers for %d experts", ld, n_experts);
     ROCML_REQUIRE(n_tokens >= 0 && n_experts > 0 && n_experts <= RT_MAX_PER_LANE * WAVE, "moe_route: %d experts (1 to %d)", n_experts,
                   RT_MAX_PER_LANE * WAVE);
     ROCML_REQUIRE(top >= 1 && top <= WAVE && top <= n_experts, "moe_route: %d chosen of %d experts", top, n_experts);
@@ -140,7 +161,8 @@ ROCML_EXPORT int rocml_moe_route(const float* logits, int n_tokens, int n_expert
     if (n_tokens == 0) return 0;
     size_t lds = (size_t)(RT_BLOCK / WAVE) * n_experts * sizeof(float);
     moe_route_kernel<<<ceil_div(n_tokens, RT_BLOCK / WAVE), RT_BLOCK, lds, stream>>>(logits, n_tokens, n_experts, top, group_count,
-                                                                                     group_keep, sum_eps, chosen, weight, bias);
+                                                                                     group_keep, sum_eps, chosen, weight, bias,
+                                                                                     sigmoid, correction, group_top2, ld);
     ROCML_CHECK_LAUNCH("moe_route");
     return 0;
 }

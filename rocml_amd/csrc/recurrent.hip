@@ -893,7 +893,7 @@ ROCML_EXPORT int rocml_mlstm_scan(const float* proj, int ld, int q_col0, int k_c
 template <typename TO>
 __global__ void __launch_bounds__(RC_BLOCK)
 head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ g, int ldg, int g_col0,
-                      const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps) {
+                      const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps, int silu) {
     int lane = threadIdx.x & (WAVE - 1);
     long long row = (long long)blockIdx.x * (RC_BLOCK / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -906,7 +906,8 @@ head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ g, 
     const float* gr = g + (size_t)t * ldg + g_col0 + (size_t)h * dv;
     for (int j = lane; j < dv; j += WAVE) {
         float gate = 1.0f / (1.0f + expf(-gr[j]));
-        Elem<TO>::store(out + (size_t)row * dv + j, src[j] * inv * gain[(size_t)h * dv + j] * gate);
+        if (silu) gate *= gr[j];
+        Elem<TO>::store(out + (size_t)row * dv + j, src[j] * inv * (gain ? gain[(size_t)h * dv + j] : 1.0f) * gate);
     }
 }
 
@@ -963,23 +964,25 @@ head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__
     }
 }
 
+// gate_act: 0 the gate is sigmoid(g), 1 it is silu(g) = g sigmoid(g).  gain may be null (ones).
 ROCML_EXPORT int rocml_head_norm_gate(const float* o, const float* g, int ldg, int g_col0, const float* gain, void* out,
-                                      int out_dtype, int n_tokens, int n_heads, int dv, float eps, hipStream_t stream) {
-    ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && dv > 0 && g_col0 >= 0 && ldg >= g_col0 + n_heads * dv && o && g && gain && out,
+                                      int out_dtype, int n_tokens, int n_heads, int dv, float eps, int gate_act, hipStream_t stream) {
+    ROCML_REQUIRE(gate_act == 0 || gate_act == 1, "head_norm_gate: unknown gate activation %d", gate_act);
+    ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && dv > 0 && g_col0 >= 0 && ldg >= g_col0 + n_heads * dv && o && g && out,
                   "head_norm_gate: bad arguments T=%d heads=%d dv=%d ld=%d", n_tokens, n_heads, dv, ldg);
     long long rows = (long long)n_tokens * n_heads;
     if (rows == 0) return 0;
     int grid = ceil_div(rows, RC_BLOCK / WAVE);
-    bool vec = dv % 4 == 0 && dv <= 8 * WAVE && ldg % 4 == 0 && g_col0 % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0 &&
+    bool vec = gate_act == 0 && gain && dv % 4 == 0 && dv <= 8 * WAVE && ldg % 4 == 0 && g_col0 % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0 &&
                (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0;
     if (vec && out_dtype == ROCML_F32)
         head_norm_gate_vec_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
     else if (vec && out_dtype == ROCML_BF16)
         head_norm_gate_vec_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
     else if (out_dtype == ROCML_F32)
-        head_norm_gate_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
+        head_norm_gate_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps, gate_act);
     else if (out_dtype == ROCML_BF16)
-        head_norm_gate_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
+        head_norm_gate_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps, gate_act);
     else return rocml_fail("head_norm_gate: unknown dtype code %d", out_dtype);
     ROCML_CHECK_LAUNCH("head_norm_gate");
     return 0;
@@ -1096,5 +1099,260 @@ ROCML_EXPORT int rocml_gated_part_norm(const float* y, const float* z, int ldz, 
         gated_part_norm_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(y, z, ldz, z_col0, gain, (bf16_t*)out, n, parts, eps);
     else return rocml_fail("gated_part_norm: unknown dtype code %d", out_dtype);
     ROCML_CHECK_LAUNCH("gated_part_norm");
+    return 0;
+}
+
+// ---- recurrences with a decay per key channel ---------------------------------------------
+// Per head a state S [dk, dv] that starts at zero, decays row by row and takes the outer product of the
+// token's key and value: S <- diag(w_t) S + k_t v_t^T.  Two ways to read it:
+//   after the update (a retention):        o_t = S_t^T q_t, with w_t one constant per head;
+//   before it, with a bonus on the token:  o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t, with w_t per token and channel.
+// The columns of S (one per value) do not depend on each other: a block takes (sequence, head, 16 values), the 16
+// lanes of a row of lanes hold one column, lane l the entries l, l + 16, ..., and add their parts of the dot product
+// with q across the row.  Four tokens are worked on at a time (all their operands are requested first).  The state
+// is stored column by column, [slot, head, dv, dk].  Everything is 32-bit.
+constexpr int DS_COLS = 16;      // values (columns of the state) per block
+constexpr int DS_LANES = 16;     // lanes that share a column
+constexpr int DS_TOKENS = 4;     // tokens in flight
+
+struct DecayScanArgs {
+    const float* q; int ldq; int q_col0;
+    const float* k; int ldk; int k_col0;
+    const float* v; int ldv; int v_col0;
+    const float* w; int ldw; int w_col0;      // per token and channel, or null
+    const float* head_decay;                   // [H], or null (then w)
+    const float* bonus;                        // [H * dk], or null: the state is read after its update
+    float* state; const int* cu_seqlens; const int* seq_slots;
+    float* out; int n_heads; int dk; int dv;
+};
+
+__device__ __forceinline__ float ds_row_sum(float v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    return v;
+}
+
+template <int R, bool BONUS>
+__global__ void __launch_bounds__(DS_COLS * DS_LANES)
+decay_scan_kernel(DecayScanArgs a) {
+    int b = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
+    int l = threadIdx.x % DS_LANES, c = threadIdx.x / DS_LANES;
+    int col = tile * DS_COLS + c;
+    bool col_ok = col < a.dv;
+    int first = a.cu_seqlens[b], n = a.cu_seqlens[b + 1] - first;
+    float* st = a.state + (((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv + (col_ok ? col : 0)) * a.dk;
+    float s[R], u[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int i = l + r * DS_LANES;
+        s[r] = (col_ok && i < a.dk) ? st[i] : 0.f;
+        u[r] = (BONUS && i < a.dk) ? a.bonus[(size_t)h * a.dk + i] : 0.f;
+    }
+    float hd = a.head_decay ? a.head_decay[h] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += DS_TOKENS) {
+        float q[DS_TOKENS][R], k[DS_TOKENS][R], w[DS_TOKENS][R], v[DS_TOKENS];
+#pragma unroll
+        for (int j = 0; j < DS_TOKENS; ++j) {
+            bool ok = t0 + j < n;
+            size_t row = (size_t)(first + (ok ? t0 + j : 0));
+            v[j] = (ok && col_ok) ? a.v[row * a.ldv + a.v_col0 + (size_t)h * a.dv + col] : 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                int i = l + r * DS_LANES;
+                bool in = ok && i < a.dk;
+                size_t e = (size_t)h * a.dk + i;
+                q[j][r] = in ? a.q[row * a.ldq + a.q_col0 + e] : 0.f;
+                k[j][r] = in ? a.k[row * a.ldk + a.k_col0 + e] : 0.f;
+                w[j][r] = a.w ? (in ? a.w[row * a.ldw + a.w_col0 + e] : 1.f) : hd;
+            }
+        }
+        float acc[DS_TOKENS];
+#pragma unroll
+        for (int j = 0; j < DS_TOKENS; ++j) {
+            float sum = 0.f;
+            if (t0 + j < n) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float kv = k[j][r] * v[j];
+                    if constexpr (BONUS) {
+                        sum = fmaf(fmaf(u[r], kv, s[r]), q[j][r], sum);
+                        s[r] = fmaf(w[j][r], s[r], kv);
+                    } else {
+                        s[r] = fmaf(w[j][r], s[r], kv);
+                        sum = fmaf(s[r], q[j][r], sum);
+                    }
+                }
+            }
+            acc[j] = sum;
+        }
+#pragma unroll
+        for (int j = 0; j < DS_TOKENS; ++j) acc[j] = ds_row_sum(acc[j]);
+        if (l < DS_TOKENS && col_ok) {
+            float mine = acc[0];
+#pragma unroll
+            for (int j = 1; j < DS_TOKENS; ++j) mine = l == j ? acc[j] : mine;
+            if (t0 + l < n) a.out[(size_t)(first + t0 + l) * a.n_heads * a.dv + (size_t)h * a.dv + col] = mine;
+        }
+    }
+    if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int i = l + r * DS_LANES;
+            if (i < a.dk) st[i] = s[r];
+        }
+    }
+}
+
+template <int R>
+static void launch_decay_scan(const DecayScanArgs& a, int n_seqs, hipStream_t stream) {
+    dim3 grid(n_seqs, a.n_heads, ceil_div(a.dv, DS_COLS));
+    if (a.bonus) decay_scan_kernel<R, true><<<grid, DS_COLS * DS_LANES, 0, stream>>>(a);
+    else decay_scan_kernel<R, false><<<grid, DS_COLS * DS_LANES, 0, stream>>>(a);
+}
+
+ROCML_EXPORT int rocml_decay_scan(const float* q, int ldq, int q_col0, const float* k, int ldk, int k_col0, const float* v,
+                                  int ldv, int v_col0, const float* w, int ldw, int w_col0, const float* head_decay,
+                                  const float* bonus, float* state, int n_slots, const int* cu_seqlens, const int* seq_slots,
+                                  int n_seqs, int n_tokens, float* out, int n_heads, int dk, int dv, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && n_slots > 0 && n_heads > 0 && dk > 0 && dv > 0, "decay_scan: bad sizes T=%d B=%d H=%d",
+                  n_tokens, n_seqs, n_heads);
+    ROCML_REQUIRE(dk <= 16 * DS_LANES, "decay_scan: a key size of %d exceeds %d", dk, 16 * DS_LANES);
+    ROCML_REQUIRE(q && k && v && state && cu_seqlens && seq_slots && out, "decay_scan: missing arguments");
+    ROCML_REQUIRE((w != nullptr) != (head_decay != nullptr), "decay_scan: a decay per token and channel or one per head, one of the two");
+    ROCML_REQUIRE(q_col0 >= 0 && k_col0 >= 0 && v_col0 >= 0 && ldq >= q_col0 + n_heads * dk && ldk >= k_col0 + n_heads * dk &&
+                      ldv >= v_col0 + n_heads * dv && (!w || (w_col0 >= 0 && ldw >= w_col0 + n_heads * dk)),
+                  "decay_scan: a row stride is too small for its columns");
+    if (n_tokens == 0 || n_seqs == 0) return 0;
+    DecayScanArgs a{q, ldq, q_col0, k, ldk, k_col0, v, ldv, v_col0, w, ldw, w_col0, head_decay, bonus, state, cu_seqlens, seq_slots,
+                    out, n_heads, dk, dv};
+    int r = ceil_div(dk, DS_LANES);
+    if (r <= 1) launch_decay_scan<1>(a, n_seqs, stream);
+    else if (r <= 2) launch_decay_scan<2>(a, n_seqs, stream);
+    else if (r <= 4) launch_decay_scan<4>(a, n_seqs, stream);
+    else if (r <= 8) launch_decay_scan<8>(a, n_seqs, stream);
+    else launch_decay_scan<16>(a, n_seqs, stream);
+    ROCML_CHECK_LAUNCH("decay_scan");
+    return 0;
+}
+
+// ---- rotation of heads inside a 32-bit matrix --------------------------------------------
+// Columns col0 .. col0 + n_heads * d - 1 of buf [T, ld]: of every head the first `rot` numbers turn, number i with
+// number i + rot/2 by the angle whose cosine and sine stand in column i of the tables [T, rot/2]; then every number
+// of the heads is multiplied by `scale`.  In place; a thread owns a pair (or one number beyond the rotated part).
+__global__ void __launch_bounds__(RC_BLOCK)
+rotate_rows_kernel(float* __restrict__ buf, int ld, int col0, int n_heads, int d, int rot, const float* __restrict__ cos_t,
+                   const float* __restrict__ sin_t, float scale, long long total) {
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    int half = rot / 2, per_head = d - half;
+    long long th = idx / per_head;
+    int e = (int)(idx - th * per_head);
+    long long t = th / n_heads;
+    int h = (int)(th - t * n_heads);
+    float* row = buf + (size_t)t * ld + col0 + (size_t)h * d;
+    if (e < half) {
+        float c = cos_t[(size_t)t * half + e], s = sin_t[(size_t)t * half + e];
+        float x = row[e], y = row[e + half];
+        row[e] = (x * c - y * s) * scale;
+        row[e + half] = (y * c + x * s) * scale;
+    } else {
+        row[e + half] *= scale;
+    }
+}
+
+ROCML_EXPORT int rocml_rotate_rows(float* buf, int ld, int col0, int n_tokens, int n_heads, int d, int rot, const float* cos_t,
+                                   const float* sin_t, float scale, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && d > 0 && rot >= 0 && rot % 2 == 0 && rot <= d, "rotate_rows: bad sizes heads=%d d=%d rot=%d",
+                  n_heads, d, rot);
+    ROCML_REQUIRE(buf && col0 >= 0 && ld >= col0 + n_heads * d && (rot == 0 || (cos_t && sin_t)), "rotate_rows: bad arguments");
+    long long total = (long long)n_tokens * n_heads * (d - rot / 2);
+    if (total == 0) return 0;
+    rotate_rows_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(buf, ld, col0, n_heads, d, rot, cos_t, sin_t, scale, total);
+    ROCML_CHECK_LAUNCH("rotate_rows");
+    return 0;
+}
+
+// ---- mixes of a token's input with the previous token's ------------------------------------
+// out[m, t, :] = h_t + (h_(t-1) - h_t) * mu[m, :] for every one of the n_mix rows of mu, in 32-bit, written in out's
+// type.  Before a sequence's first token of the step stands the sequence's kept row (state [slot, n], zeros at its
+// start); the thread that reads it also writes the sequence's last row of the step there, so nobody reads a row
+// that another thread has replaced.
+template <typename T>
+__global__ void __launch_bounds__(RC_BLOCK)
+shift_mix_kernel(const T* __restrict__ h, int n, const float* __restrict__ mu, int n_mix, float* __restrict__ state,
+                 const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots,
+                 T* __restrict__ out, long long total, long long mix_stride) {
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / n;
+    int c = (int)(idx - t * n);
+    int b = token_seq[t];
+    int first = cu_seqlens[b];
+    float cur = Elem<T>::load(h + idx), prev;
+    if (t == first) {
+        float* st = state + (size_t)seq_slots[b] * n + c;
+        prev = *st;
+        *st = Elem<T>::load(h + (size_t)(cu_seqlens[b + 1] - 1) * n + c);
+    } else {
+        prev = Elem<T>::load(h + idx - n);
+    }
+    float d = prev - cur;
+    for (int m = 0; m < n_mix; ++m) Elem<T>::store(out + m * mix_stride + idx, fmaf(d, mu[(size_t)m * n + c], cur));
+}
+
+ROCML_EXPORT int rocml_shift_mix(const void* h, int dtype, int n_tokens, int n, const float* mu, int n_mix, float* state, int n_slots,
+                                 const int* token_seq, const int* cu_seqlens, const int* seq_slots, int n_seqs, void* out,
+                                 hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && n > 0 && n_mix > 0 && n_slots > 0 && n_seqs >= 0, "shift_mix: bad sizes T=%d n=%d mixes=%d", n_tokens, n, n_mix);
+    ROCML_REQUIRE(h && mu && state && token_seq && cu_seqlens && seq_slots && out, "shift_mix: missing arguments");
+    long long total = (long long)n_tokens * n;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, RC_BLOCK);
+    if (dtype == ROCML_F32)
+        shift_mix_kernel<float><<<grid, RC_BLOCK, 0, stream>>>((const float*)h, n, mu, n_mix, state, token_seq, cu_seqlens, seq_slots,
+                                                             (float*)out, total, total);
+    else if (dtype == ROCML_BF16)
+        shift_mix_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>((const bf16_t*)h, n, mu, n_mix, state, token_seq, cu_seqlens, seq_slots,
+                                                              (bf16_t*)out, total, total);
+    else return rocml_fail("shift_mix: unknown dtype code %d", dtype);
+    ROCML_CHECK_LAUNCH("shift_mix");
+    return 0;
+}
+
+// ---- small maps between two products ------------------------------------------------------
+// out = tanh(x) in out's type (the middle of a decay's two small matrices), and
+// out = exp(-exp(x + offset[c])) in 32-bit (the decay itself, per token and channel).
+template <typename T>
+__global__ void __launch_bounds__(RC_BLOCK)
+tanh_kernel(const float* __restrict__ x, T* __restrict__ out, long long total) {
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx < total) Elem<T>::store(out + idx, tanhf(x[idx]));
+}
+
+ROCML_EXPORT int rocml_tanh(const float* x, void* out, int out_dtype, long long total, hipStream_t stream) {
+    ROCML_REQUIRE(total >= 0 && x && out, "tanh: bad arguments");
+    if (total == 0) return 0;
+    int grid = ceil_div(total, RC_BLOCK);
+    if (out_dtype == ROCML_F32) tanh_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(x, (float*)out, total);
+    else if (out_dtype == ROCML_BF16) tanh_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(x, (bf16_t*)out, total);
+    else return rocml_fail("tanh: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("tanh");
+    return 0;
+}
+
+__global__ void __launch_bounds__(RC_BLOCK)
+double_exp_decay_kernel(float* __restrict__ x, const float* __restrict__ offset, int n, long long total) {
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx < total) x[idx] = expf(-expf(x[idx] + offset[idx % n]));
+}
+
+ROCML_EXPORT int rocml_double_exp_decay(float* x, const float* offset, int n_rows, int n, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0 && x && offset, "double_exp_decay: bad arguments");
+    long long total = (long long)n_rows * n;
+    if (total == 0) return 0;
+    double_exp_decay_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(x, offset, n, total);
+    ROCML_CHECK_LAUNCH("double_exp_decay");
     return 0;
 }

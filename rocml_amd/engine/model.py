@@ -151,7 +151,8 @@ class DecoderModel:
         rows of logits asks the workspace for: the residual stream, the largest layer's buffers
         (layers share theirs), the wanted rows and their logits, and the scratch memory."""
         per_layer = max(b.activation_bytes(n_tokens) for b in self.blocks)
-        return (n_tokens * self.spec.hidden * 4 + per_layer + self.head.activation_bytes(n_wanted)
+        kept = n_tokens * self.spec.hidden * 4 if any(e.add_embedding for e in self.spec.schedule) else 0
+        return (kept + n_tokens * self.spec.hidden * 4 + per_layer + self.head.activation_bytes(n_wanted)
                 + Workspace.SCRATCH_BYTES)
 
     def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None,
@@ -182,6 +183,11 @@ class DecoderModel:
         step.tables = self.tables
         x = ws.get("model.x", (step.n_tokens, s.hidden), torch.float32)
         self.embedding.forward(step, x)
+        x0 = None
+        if any(e.add_embedding for e in s.schedule):
+            # entries that add the embedding's output to the stream later need it kept
+            x0 = ws.get("model.x0", (step.n_tokens, s.hidden), torch.float32)
+            ops.weighted_sum(x0, [x], [1.0])
         for i, entry in enumerate(s.schedule):
             owner = i if entry.reads_cache_of is None else entry.reads_cache_of
             view = cache.view(owner, step) if cache.has_line(owner) else None
@@ -189,12 +195,14 @@ class DecoderModel:
             if entry.offset_row is not None:
                 # (sums that a product left for the next norm may still be missing from x: additions commute)
                 ops.add_row_vector(x, self.pass_offset[entry.offset_row])
+            if entry.add_embedding:
+                ops.add_into(x, x0)
             if not getattr(block, "takes_pending", False):
                 ws.flush_pending()
             # the block that runs next may let this block's last product prepare its first norm
             following = self.blocks[s.schedule[i + 1].layer] if i + 1 < len(s.schedule) else None
             hint = None
-            if following is not None and s.schedule[i + 1].offset_row is not None:
+            if following is not None and (s.schedule[i + 1].offset_row is not None or s.schedule[i + 1].add_embedding):
                 following = None      # the stream changes between the two blocks: nothing can be prepared across
             if getattr(block, "takes_next_norm", False) and hasattr(following, "entry_hint"):
                 hint = following.entry_hint(step)

@@ -49,6 +49,9 @@ _SIGNATURES = {
         "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _I, _P],
         "rocml_sum_norm": [_P, _I, _I, _F, _F, _I, _P, _P, _P, _F, _P, _I, _P],
         "rocml_convert": [_P, _P, _I, _LL, _P],
+        "rocml_softcap": [_P, _F, _LL, _P],
+        "rocml_weighted_sum": [_P, _P, _P, _I, _F, _LL, _P],
+        "rocml_row_gate_add": [_P, _P, _P, _I, _I, _I, _P],
     },
     "recurrent": {
         "rocml_causal_conv": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _P],
@@ -56,10 +59,15 @@ _SIGNATURES = {
         "rocml_gated_part_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
         "rocml_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _F, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
         "rocml_mlstm_tile": [],
-        "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+        "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
+        "rocml_decay_scan": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
+        "rocml_rotate_rows": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P],
+        "rocml_shift_mix": [_P, _I, _I, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P],
+        "rocml_tanh": [_P, _P, _I, _LL, _P],
+        "rocml_double_exp_decay": [_P, _P, _I, _I, _P],
     },
     "moe": {
-        "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P, _P],
+        "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P, _I, _P, _I, _I, _P],
         "rocml_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _I, _P],
         "rocml_moe_gemm": [_P, _I, _I, _I, _P, _I, _P, _P, _I, _LL, _I, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
         "rocml_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
@@ -73,7 +81,7 @@ _SIGNATURES = {
     },
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
-                            _P, _I, _I, _P, _I, _I, _P, _LL, _I, _I, _I, _P, _I, _P],
+                            _P, _I, _I, _P, _I, _I, _P, _LL, _I, _I, _I, _P, _I, _P, _F, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
                                          _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P, _I, _P, _I, _P],
         "rocml_attention_prefill_fused": [_P, _I, _P, _F, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I,
@@ -622,6 +630,43 @@ def convert(x: torch.Tensor, out: torch.Tensor) -> None:
     _check("elementwise", library("elementwise").rocml_convert(_ptr(x), _ptr(out), _code(out), x.numel(), _stream()))
 
 
+def softcap(x: torch.Tensor, cap: float) -> None:
+    """``x <- cap * tanh(x / cap)`` in place, 32-bit."""
+    _dev(x)
+    _want(x, torch.float32, "the values to cap")
+    _check("elementwise", library("elementwise").rocml_softcap(_ptr(x), float(cap), x.numel(), _stream()))
+
+
+def weighted_sum(out: torch.Tensor, branches: Sequence[torch.Tensor], weights: Sequence[float], alpha: float = 0.0) -> None:
+    """``out <- alpha * out + sum_b weights[b] * branches[b]``, all 32-bit and of one shape."""
+    _dev(out, *branches)
+    if not 1 <= len(branches) <= 4 or len(weights) != len(branches):
+        raise KernelError("weighted_sum takes one to four branches and a weight for each")
+    for y in (out, *branches):
+        _want(y, torch.float32, "a summand")
+        if y.shape != out.shape:
+            raise KernelError("weighted_sum: shapes differ")
+    ys = (ctypes.c_void_p * len(branches))(*[y.data_ptr() for y in branches])
+    ws = (ctypes.c_float * len(branches))(*[float(w) for w in weights])
+    _check("elementwise", library("elementwise").rocml_weighted_sum(_ptr(out), ys, ws, len(branches), float(alpha), out.numel(),
+                                                                   _stream()))
+
+
+def row_gate_add(x: torch.Tensor, y: torch.Tensor, gate: torch.Tensor) -> None:
+    """``x[t] += sigmoid(gate[t]) * y[t]`` for 32-bit ``x``, ``y [T, n]`` and one 32-bit gate logit per row (a column
+    of a matrix: ``gate [T, 1]`` with any row stride)."""
+    _dev(x, y)
+    if not gate.is_cuda:
+        raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
+    for t, what in ((x, "the stream"), (y, "the summand"), (gate, "the gate")):
+        _want(t, torch.float32, what)
+    rows, n = x.shape
+    if y.shape != x.shape or gate.dim() != 2 or gate.shape != (rows, 1):
+        raise KernelError("row_gate_add: sizes differ")
+    _check("elementwise", library("elementwise").rocml_row_gate_add(_ptr(x), _ptr(y), _ptr(gate), max(gate.stride(0), 1), rows, n,
+                                                                   _stream()))
+
+
 def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
     _dev(x, y)
     _want(x, torch.float32, "residual")
@@ -785,7 +830,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
               cu_seqlens: Optional[torch.Tensor] = None, max_new: int = 0,
               q_counts: Optional[Sequence[int]] = None, max_len: int = 0, n_splits: int = 0,
               v_head_dim: Optional[int] = None, values_in_keys: bool = False, chunk: Optional[int] = None,
-              slopes: Optional[torch.Tensor] = None, sink: bool = False) -> None:
+              slopes: Optional[torch.Tensor] = None, sink: bool = False, sinks: Optional[torch.Tensor] = None,
+              softcap: Optional[float] = None) -> None:
     """Attention of the step's query tokens over the cache.  Keys are ``[pages, Hkv, page, D]``,
     values ``[pages, Hkv, D, page]``.  ``cu_seqlens`` (device), ``q_counts`` (the same knowledge on
     the host: query tokens of each sequence), ``max_new`` (the most of them) and ``max_len``
@@ -796,8 +842,15 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
     row.  ``chunk``: blocks of so many positions, counted from 0, instead of a window: a query sees
     its own block up to itself.  ``slopes`` (32-bit, one per query head): ``slope * (i - j)`` is
     taken off the score of query ``i`` and key ``j``.  ``sink``: the denominator of the softmax has
-    one more term ``exp(0)``."""
-    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens, slopes)
+    one more term ``exp(0)``, or with ``sinks`` (32-bit, one per query head) ``exp(sinks[h])``.
+    ``softcap``: the scaled score ``s`` becomes ``softcap * tanh(s / softcap)`` before the mask."""
+    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens, slopes, sinks)
+    if sinks is not None:
+        _want(sinks, torch.float32, "sinks")
+        if sinks.numel() != n_heads or not sink:
+            raise KernelError("one sink per query head is needed, and the sink switched on")
+    if softcap is not None and not softcap > 0:
+        raise KernelError(f"the soft cap of the scores must be positive, got {softcap}")
     n_tokens = q.shape[0]
     dv = head_dim if v_head_dim is None else int(v_head_dim)
     if q.shape != (n_tokens, n_heads * head_dim) or out.shape != (n_tokens, n_heads * dv) or out.dtype != q.dtype:
@@ -836,7 +889,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
         block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
         page, scale, 0 if window is None else int(window), algo, _ptr(cu_seqlens), n_seqs, max_new,
         counts, max_len, n_splits, ws_ptr, ws_bytes, dv, 1 if values_in_keys else 0,
-        0 if chunk is None else int(chunk), _ptr(slopes), 1 if sink else 0, _stream()))
+        0 if chunk is None else int(chunk), _ptr(slopes), 1 if sink else 0, _ptr(sinks),
+        0.0 if softcap is None else float(softcap), _stream()))
 
 
 FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)
@@ -1168,19 +1222,110 @@ def mlstm_scan(proj: torch.Tensor, q_col0: int, k_col0: int, v_col0: int, i_col0
         n_seqs, n_tokens, _ptr(out), n_heads, head_dim, v_head_dim, _stream()))
 
 
-def head_norm_gate(o: torch.Tensor, g: torch.Tensor, g_col0: int, gain: torch.Tensor, out: torch.Tensor, n_heads: int,
-                   eps: float) -> None:
-    """``out = rms_heads(o) * gain * sigmoid(g)``: every one of the ``n_heads`` equal parts of a row of the 32-bit
-    ``o [T, n]`` divided by its own root mean square; ``g`` is columns ``g_col0 ..`` of a 32-bit matrix."""
+HEAD_GATES = {"sigmoid": 0, "silu": 1}
+
+
+def head_norm_gate(o: torch.Tensor, g: torch.Tensor, g_col0: int, gain: Optional[torch.Tensor], out: torch.Tensor, n_heads: int,
+                   eps: float, gate: str = "sigmoid") -> None:
+    """``out = rms_heads(o) * gain * act(g)``: every one of the ``n_heads`` equal parts of a row of the 32-bit
+    ``o [T, n]`` divided by its own root mean square; ``g`` is columns ``g_col0 ..`` of a 32-bit matrix; ``act`` is
+    ``sigmoid`` or ``silu``; without ``gain`` the normed values are only gated."""
     _dev(o, g, gain, out)
-    for t, what in ((o, "norm input"), (g, "gate"), (gain, "norm gain")):
+    for t, what in ((o, "norm input"), (g, "gate")) + (((gain, "norm gain"),) if gain is not None else ()):
         _want(t, torch.float32, what)
+    if gate not in HEAD_GATES:
+        raise KernelError(f"unknown gate {gate!r}; known: {sorted(HEAD_GATES)}")
     rows, n = o.shape
-    if n % n_heads != 0 or gain.numel() != n or out.shape != o.shape or g.shape[0] != rows or g.shape[1] < g_col0 + n:
+    if n % n_heads != 0 or (gain is not None and gain.numel() != n) or out.shape != o.shape or g.shape[0] != rows \
+            or g.shape[1] < g_col0 + n:
         raise KernelError("head_norm_gate: sizes differ")
     _check("recurrent", library("recurrent").rocml_head_norm_gate(
         _ptr(o), _ptr(g), g.shape[1], g_col0, _ptr(gain), _ptr(out), _code(out), rows, n_heads, n // n_heads, float(eps),
-        _stream()))
+        HEAD_GATES[gate], _stream()))
+
+
+def decay_scan(q: torch.Tensor, q_col0: int, k: torch.Tensor, k_col0: int, v: torch.Tensor, v_col0: int,
+               state: torch.Tensor, cu_seqlens: torch.Tensor, seq_slots: torch.Tensor, out: torch.Tensor,
+               n_heads: int, head_dim: int, v_head_dim: int, head_decay: Optional[torch.Tensor] = None,
+               decay: Optional[torch.Tensor] = None, decay_col0: int = 0, bonus: Optional[torch.Tensor] = None) -> None:
+    """A recurrence whose state per head, ``S [dk, dv]``, decays row by row, over the step's tokens, per sequence in
+    order: ``S <- diag(w_t) S + k_t v_t^T``.  With ``head_decay`` (one number per head) ``w_t`` is that constant and
+    the output reads the new state, ``o_t = S_t^T q_t``; with ``decay`` (per token and key channel, columns
+    ``decay_col0 ..`` of a 32-bit matrix) and ``bonus`` ``u [H * dk]`` the output reads the state before the update,
+    ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t``.  q, k, v are column ranges of 32-bit matrices ``[T, ld]``;
+    ``state [slots, H, dv, dk]``; ``out [T, H * dv]``; all 32-bit."""
+    _dev(q, k, v, state, cu_seqlens, seq_slots, out, head_decay, decay, bonus)
+    for t, what in ((q, "queries"), (k, "keys"), (v, "values"), (state, "recurrent state"), (out, "recurrence output")):
+        _want(t, torch.float32, what)
+    n_tokens, n_seqs = out.shape[0], seq_slots.numel()
+    if state.dim() != 4 or state.shape[1:] != (n_heads, v_head_dim, head_dim):
+        raise KernelError(f"recurrent state {tuple(state.shape)} does not fit {n_heads} heads of {head_dim} x {v_head_dim}")
+    if out.shape != (n_tokens, n_heads * v_head_dim) or cu_seqlens.numel() != n_seqs + 1 \
+            or any(t.dim() != 2 or t.shape[0] != n_tokens for t in (q, k, v)):
+        raise KernelError("recurrence inputs, output or tables do not fit the step")
+    if (head_decay is None) == (decay is None) or (decay is None) != (bonus is None):
+        raise KernelError("the recurrence takes one decay per head, or a decay per token and channel together with a bonus")
+    for t, n, what in ((head_decay, n_heads, "the heads' decays"), (bonus, n_heads * head_dim, "the bonus")):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != n):
+            raise KernelError(f"{what} must be 32-bit with {n} numbers")
+    if decay is not None and (decay.dtype != torch.float32 or decay.dim() != 2 or decay.shape[0] != n_tokens):
+        raise KernelError("the decays per token must be a 32-bit matrix with a row per token")
+    _check("recurrent", library("recurrent").rocml_decay_scan(
+        _ptr(q), q.shape[1], q_col0, _ptr(k), k.shape[1], k_col0, _ptr(v), v.shape[1], v_col0, _ptr(decay),
+        0 if decay is None else decay.shape[1], decay_col0, _ptr(head_decay), _ptr(bonus), _ptr(state), state.shape[0],
+        _ptr(cu_seqlens), _ptr(seq_slots), n_seqs, n_tokens, _ptr(out), n_heads, head_dim, v_head_dim, _stream()))
+
+
+def rotate_rows(buf: torch.Tensor, col0: int, n_heads: int, head_dim: int, rot_dim: int, cos: Optional[torch.Tensor],
+                sin: Optional[torch.Tensor], scale: float = 1.0) -> None:
+    """In place on columns ``col0 .. col0 + n_heads * head_dim - 1`` of the 32-bit ``buf [T, ld]``: of every head the
+    first ``rot_dim`` numbers turn (number ``i`` with ``i + rot_dim / 2``, angles from the tables ``[T, rot_dim / 2]``),
+    then the heads are multiplied by ``scale``."""
+    _dev(buf, cos, sin)
+    _want(buf, torch.float32, "the matrix to rotate")
+    n_tokens = buf.shape[0]
+    if rot_dim:
+        if cos is None or sin is None or cos.shape != (n_tokens, rot_dim // 2) or sin.shape != cos.shape:
+            raise KernelError(f"rotation tables must be {(n_tokens, rot_dim // 2)}")
+    _check("recurrent", library("recurrent").rocml_rotate_rows(_ptr(buf), buf.shape[1], col0, n_tokens, n_heads, head_dim, rot_dim,
+                                                             _ptr(cos), _ptr(sin), float(scale), _stream()))
+
+
+def shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor,
+              seq_slots: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[m, t] = h_t + (h_(t-1) - h_t) * mu[m]`` for every row of the 32-bit ``mu [mixes, n]``, in 32-bit, written in
+    ``h``'s type.  Before a sequence's first token of the step stands its kept row ``state [slots, n]`` (32-bit, zeros
+    at its start), which is replaced by the sequence's last row of the step."""
+    _dev(h, mu, state, token_seq, cu_seqlens, seq_slots, out)
+    _want(mu, torch.float32, "mix weights")
+    _want(state, torch.float32, "the kept row")
+    n_tokens, n = h.shape
+    n_seqs = seq_slots.numel()
+    if mu.dim() != 2 or mu.shape[1] != n or out.shape != (mu.shape[0], n_tokens, n) or out.dtype != h.dtype \
+            or state.dim() != 2 or state.shape[1] != n or token_seq.numel() != n_tokens or cu_seqlens.numel() != n_seqs + 1:
+        raise KernelError("shift_mix: sizes differ")
+    _check("recurrent", library("recurrent").rocml_shift_mix(
+        _ptr(h), _code(h), n_tokens, n, _ptr(mu), mu.shape[0], _ptr(state), state.shape[0], _ptr(token_seq), _ptr(cu_seqlens),
+        _ptr(seq_slots), n_seqs, _ptr(out), _stream()))
+
+
+def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = tanh(x)`` in ``out``'s type, for 32-bit ``x``."""
+    _dev(x, out)
+    _want(x, torch.float32, "the values")
+    if x.numel() != out.numel():
+        raise KernelError("tanh: sizes differ")
+    _check("recurrent", library("recurrent").rocml_tanh(_ptr(x), _ptr(out), _code(out), x.numel(), _stream()))
+
+
+def double_exp_decay(x: torch.Tensor, offset: torch.Tensor) -> None:
+    """``x <- exp(-exp(x + offset))`` in place for the 32-bit ``x [T, n]`` and ``offset [n]``."""
+    _dev(x, offset)
+    _want(x, torch.float32, "decay logits")
+    _want(offset, torch.float32, "decay offsets")
+    if x.dim() != 2 or offset.numel() != x.shape[1]:
+        raise KernelError("double_exp_decay: sizes differ")
+    _check("recurrent", library("recurrent").rocml_double_exp_decay(_ptr(x), _ptr(offset), x.shape[0], x.shape[1], _stream()))
 
 
 # ---- experts -----------------------------------------------------------------------------
@@ -1193,12 +1338,20 @@ def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
 
 
 def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: torch.Tensor, weight: torch.Tensor,
-              bias: Optional[torch.Tensor] = None) -> None:
+              bias: Optional[torch.Tensor] = None, sigmoid: bool = False, correction: Optional[torch.Tensor] = None,
+              group_top2: bool = False) -> None:
     """Softmax over all experts, the ``top`` best (of the experts of the ``groups[1]`` best of
     ``groups[0]`` equal groups of neighbours, a group's score being its largest, if ``groups`` is
     given), weights = chosen scores / (their sum + ``sum_eps``).  ``chosen`` int32, ``weight`` float32,
-    both ``[T, top]``.  ``bias``: 32-bit, one number per expert, added to the logits first."""
-    _dev(logits, chosen, weight, bias)
+    both ``[T, top]``.  ``bias``: 32-bit, one number per expert, added to the logits first.  ``sigmoid``: an
+    expert's score is ``sigmoid(logit)`` instead of the softmax.  ``correction``: 32-bit, one number per expert,
+    added to the scores for the choice of groups and experts only.  ``group_top2``: a group's score is the sum of
+    its two largest (corrected) scores."""
+    _dev(chosen, weight, bias, correction)
+    if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("the router's logits must be a GPU matrix with unit inner stride (rows may be the leading columns of a wider one)")
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != logits.shape[1]):
+        raise KernelError("the correction of the experts' scores must be 32-bit with one number per expert")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != logits.shape[1]):
         raise KernelError("the router's bias must be 32-bit with one number per expert")
     _want(logits, torch.float32, "router logits")
@@ -1209,7 +1362,9 @@ def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: to
         raise KernelError("moe_route: outputs must be [tokens, top]")
     count, keep = (0, 0) if groups is None else (int(groups[0]), int(groups[1]))
     _check("moe", library("moe").rocml_moe_route(_ptr(logits), n_tokens, n_experts, top, count, keep, float(sum_eps),
-                                                 _ptr(chosen), _ptr(weight), _ptr(bias), _stream()))
+                                                 _ptr(chosen), _ptr(weight), _ptr(bias), 1 if sigmoid else 0,
+                                                 _ptr(correction), 1 if group_top2 else 0,
+                                                 logits.stride(0) if n_tokens > 1 else max(logits.stride(0), n_experts), _stream()))
 
 
 def moe_plan(chosen: torch.Tensor, n_experts: int, plan: torch.Tensor):

@@ -3,7 +3,7 @@ from .base import (BuildContext, CompositeRequest, Embedding, FeedForward, Head,
 from .registry import (build_block, build_embedding, build_feed_forward, build_head, build_mixer, build_norm,
                        build_position, register_block, register_embedding, register_feed_forward,
                        register_head, register_mixer, register_norm, register_position)
-from . import rmsnorm, layernorm, rope, attention, latent_attention, state_space, matrix_memory, parallel, mlp, moe, token_side, block, embedding, head  # noqa: F401  (register the built-in parts)
+from . import rmsnorm, layernorm, rope, attention, latent_attention, state_space, matrix_memory, retention, time_mix, parallel, mlp, moe, token_side, block, embedding, head  # noqa: F401  (register the built-in parts)
 
 __all__ = ["BuildContext", "CompositeRequest", "Embedding", "FeedForward", "Head", "KVCacheRequest", "LatentCacheRequest", "Mixer", "Norm", "ParamSpec",
            "Part", "PositionEncoding", "StateRequest", "build_block", "build_embedding", "build_feed_forward",

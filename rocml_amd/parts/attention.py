@@ -13,6 +13,12 @@ blocks of positions instead of a window, a penalty on distance (a slope per head
 the softmax.  Any of these takes the layer off the matrix-core attention kernels, which know none
 of them, and onto the plain kernel, which takes them all as parameters; the projections and the
 append kernel are the same ones.
+
+Further options: a learned sink per head (``exp(sink_h)`` in the denominator), a soft cap on the scaled
+scores, and a short causal convolution per channel on q, k and v right behind their projection (32-bit, with
+the last ``taps - 1`` projected rows of a sequence kept as a state beside its keys and values).  The
+matrix-core kernels take the first two; the convolution is a kernel of its own in front of the
+norm-and-rotation kernel.
 """
 from __future__ import annotations
 
@@ -23,7 +29,7 @@ import torch
 from .. import ops
 from ..config.spec import AttentionSpec
 from ..errors import ConfigError
-from .base import BuildContext, KVCacheRequest, Mixer, ParamSpec
+from .base import BuildContext, CompositeRequest, KVCacheRequest, Mixer, ParamSpec, StateRequest
 from .registry import build_position, register_mixer
 from .residual import stream
 
@@ -55,13 +61,25 @@ class Attention(Mixer):
         self.v_head_dim = spec.head_dim if spec.v_head_dim is None else spec.v_head_dim
         # what the matrix-core kernels do not know: such a layer runs the plain attention kernel
         self.extras = (self.v_head_dim != spec.head_dim or spec.chunk is not None
-                       or spec.distance_slopes is not None or spec.sink)
+                       or spec.distance_slopes is not None or spec.sink or getattr(spec, "softcap", None) is not None)
+        self.sink_learned = bool(getattr(spec, "sink_learned", False))
+        if self.sink_learned and not spec.sink:
+            raise ConfigError("learned sinks need the sink switched on")
+        self.softcap = getattr(spec, "softcap", None)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ConfigError(f"the soft cap of the scores must be positive, got {self.softcap}")
+        self.conv = getattr(spec, "conv", None)
+        if self.conv is not None and not 1 <= self.conv <= 8:
+            raise ConfigError(f"the convolution on q, k and v has {self.conv} taps; 1 to 8 are supported")
+        if self.conv is not None and (spec.bias or spec.qk_norm is not None and getattr(spec, "qk_norm_span", "head") != "head"):
+            raise ConfigError("a convolution on q, k and v goes without biases and without a norm over the whole projection")
         if spec.q_temp is not None and not (spec.q_temp[1] > 0):
             raise ConfigError(f"the period of the query's stretch must be positive, got {spec.q_temp[1]}")
         # what only the norm-and-rotation kernel knows (the kernels that prepare their queries
         # themselves do not): a stretch of the query with its position, an output gate
         # (and a norm over a token's whole q and k rows, whose factors a kernel of their own forms first)
-        self.separate_q = spec.q_temp is not None or spec.gate or self.span == "projection"
+        self.separate_q = spec.q_temp is not None or spec.gate or self.span == "projection" or self.conv is not None \
+            or self.sink_learned or self.softcap is not None
         self.gate_per_head = bool(getattr(spec, "gate_per_head", False))
         if self.gate_per_head and not spec.gate:
             raise ConfigError("a gate per head needs the output gate switched on")
@@ -92,6 +110,10 @@ class Attention(Mixer):
         self.k_gain: Optional[torch.Tensor] = None
         self.b_qkv: Optional[torch.Tensor] = None
         self.b_o: Optional[torch.Tensor] = None
+        self.sinks: Optional[torch.Tensor] = None
+        self.conv_w: Optional[torch.Tensor] = None
+        if self.conv is not None:
+            self.kernel_families = ("recurrent",)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         s = self.spec
@@ -111,6 +133,12 @@ class Attention(Mixer):
             specs["k_norm.weight"] = ParamSpec((self.kv_dim if whole else s.head_dim,), role="gain", init="gain")
         if s.gate:
             specs["g_proj.weight"] = ParamSpec((self.g_dim, s.hidden))
+        if self.sink_learned:
+            specs["sink"] = ParamSpec((s.n_heads,), role="gain", init="normal")
+        if self.conv is not None:       # stored [channels, taps], the last tap the current token's
+            specs["q_conv.weight"] = ParamSpec((self.q_dim, self.conv), role="gain", init="normal")
+            specs["k_conv.weight"] = ParamSpec((self.kv_dim, self.conv), role="gain", init="normal")
+            specs["v_conv.weight"] = ParamSpec((self.v_dim, self.conv), role="gain", init="normal")
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -127,6 +155,11 @@ class Attention(Mixer):
                                    ).contiguous()
         if self.o_bias:
             self.b_o = tensors["o_proj.bias"]
+        if self.sink_learned:
+            self.sinks = tensors["sink"]
+        if self.conv is not None:
+            # [taps, channels] over q, k and v side by side, as the convolution kernel reads it
+            self.conv_w = torch.cat([tensors["q_conv.weight"], tensors["k_conv.weight"], tensors["v_conv.weight"]], dim=0).t().contiguous()
         if self.spec.qk_norm is not None:
             if self.norm_learned:
                 self.q_gain = tensors["q_norm.weight"]
@@ -172,11 +205,16 @@ class Attention(Mixer):
         # only the decode kernel that reads the projection's sums itself applies a scale to them
         return self._fused_decode(step)
 
-    def cache_request(self) -> KVCacheRequest:
+    def cache_request(self):
         s = self.spec
         if s.v_head_dim is None and s.chunk is None:
-            return KVCacheRequest(s.n_kv_heads, s.head_dim, s.window)
-        return KVCacheRequest(s.n_kv_heads, s.head_dim, s.window, v_head_dim=self.v_head_dim, chunk=s.chunk)
+            kv = KVCacheRequest(s.n_kv_heads, s.head_dim, s.window)
+        else:
+            kv = KVCacheRequest(s.n_kv_heads, s.head_dim, s.window, v_head_dim=self.v_head_dim, chunk=s.chunk)
+        if self.conv is None or self.conv == 1:
+            return kv
+        # the convolution's last taps - 1 inputs live beside the keys and values
+        return CompositeRequest((kv, StateRequest((self.conv - 1, self.q_dim + self.kv_dim + self.v_dim))))
 
     def _decode_splits(self, step, cache) -> int:
         """Splits of the key range in a decode step: enough blocks to fill the chip, at most one
@@ -201,6 +239,11 @@ class Attention(Mixer):
         rows = self.q_dim + self.kv_dim + self.v_dim + self.g_dim if owns_cache else self.q_dim
         if s.gate and not owns_cache:
             raise ConfigError("a gated attention layer that reads another layer's cache is not supported")
+        conv_state = None
+        if isinstance(getattr(cache, "parts", None), tuple) and cache.parts:
+            cache, conv_state = cache.parts
+        if self.conv is not None and not owns_cache:
+            raise ConfigError("an attention layer with a convolution on q, k and v cannot read another layer's cache")
         scratch = ws.scratch()
         if projected is not None:
             qkv, first = projected
@@ -212,10 +255,22 @@ class Attention(Mixer):
             # (the decode kernel that reads the projection adds four partial sums in one trip to memory
             # and further ones one after the other: K is cut into few pieces for it)
             # (the gate's columns are read where they lie: the product is then completed)
-            splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate and self.span == "head",
+            splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch,
+                              defer=not s.gate and self.span == "head" and self.conv is None,
                               max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
         if splits:      # the product's split-K partial sums; the next kernel adds them
             qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
+        if self.conv is not None:
+            # q, k and v pass the convolution in 32-bit, channel by channel; what follows reads its output
+            channels = self.q_dim + self.kv_dim + self.v_dim
+            mixed = ws.get("attn.qkv_conv", (n, channels), torch.float32)
+            if self.conv > 1:
+                kept = conv_state.state
+            else:
+                kept = ws.get("attn.no_conv_state", (1, 0, channels), torch.float32)
+            ops.causal_conv(qkv, 0, channels, self.conv_w, None, kept, step.token_seq, step.cu_seqlens, step.seq_slots, mixed,
+                            silu=False)
+            qkv = mixed
         cos = sin = None
         rot = 0
         if self.position is not None:
@@ -268,7 +323,8 @@ class Attention(Mixer):
                               s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                               cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                               max_len=step.max_len, n_splits=self._decode_splits(step, cache),
-                              v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink)
+                              v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink, sinks=self.sinks,
+                              softcap=self.softcap)
         if s.gate:
             ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:rows], group=self.v_head_dim if self.gate_per_head else 1)
         if self.b_o is not None:

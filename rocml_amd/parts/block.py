@@ -314,3 +314,74 @@ class SublayerNormBlock(Part):
 
 
 register_block("sublayer_norm", SublayerNormBlock)
+
+
+class SandwichNormBlock(Part):
+    """``x += out_norm1(mixer(norm1(x)))``, ``x += out_norm2(ffn(norm2(x)))``: a norm before and one after every
+    sublayer (the feed-forward may be absent).  The first norm of a sublayer writes the products' operand in the
+    compute type; the sublayer writes its result to a buffer of the block; one kernel then norms that buffer and
+    adds it to the 32-bit stream (it takes a product's K pieces in place of the buffer).  The norms are
+    root-mean-square norms with a gain."""
+    takes_pending = False
+    takes_next_norm = False
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        if spec.mixer_out_norm is None or (spec.ffn is not None and (spec.ffn_norm is None or spec.ffn_out_norm is None)):
+            raise ConfigError("a block with a norm before and after every sublayer needs both norms of each")
+        self.dtype = ctx.dtype
+        self.hidden = spec.mixer_norm.size
+        self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
+                         "mixer": build_mixer(spec.mixer, ctx),
+                         "mixer_out_norm": build_norm(spec.mixer_out_norm, ctx)}
+        if spec.ffn is not None:
+            self.children["ffn_norm"] = build_norm(spec.ffn_norm, ctx)
+            self.children["ffn"] = build_feed_forward(spec.ffn, ctx)
+            self.children["ffn_out_norm"] = build_norm(spec.ffn_out_norm, ctx)
+        self.mixer = self.children["mixer"]
+        self.ffn = self.children.get("ffn")
+        for name in ("mixer_out_norm", "ffn_out_norm"):
+            norm = self.children.get(name)
+            if norm is not None and (not hasattr(norm, "gain") or not hasattr(norm, "eps") or getattr(norm, "centred", False)):
+                raise ConfigError("a block that norms its sublayers' outputs before adding them needs root-mean-square norms there")
+        self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
+        self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
+        self.kernel_families = tuple(f for c in self.children.values() for f in getattr(c, "kernel_families", ()))
+
+    param_specs = PreNormBlock.param_specs
+    bind = PreNormBlock.bind
+    cache_request = PreNormBlock.cache_request
+    flops = PreNormBlock.flops
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * self.hidden * (size + 4) + self.mixer.activation_bytes(n_tokens) + \
+            (self.ffn.activation_bytes(n_tokens) if self.ffn is not None else 0)
+
+    def _sublayer(self, step, x, norm, run, out_norm) -> None:
+        ws = step.workspace
+        rs = stream(step)
+        xn = ws.get("block.xn", tuple(x.shape), self.dtype)
+        norm.forward(x, xn)
+        y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
+        rs.overwrite = rs.defer_overwrite = True
+        run(xn, y)
+        # (a product cut along K may have left its pieces for this kernel to add: they are all of y then)
+        pending = ws.take_pending_or_whole(y)
+        partials, replace = pending if pending is not None else (None, False)
+        ops.norm_add(x, y, out_norm.gain, None, out_norm.eps, layer=False, partials=partials, replace=replace)
+
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+        rs = stream(step)
+        step.workspace.flush_pending()
+        rs.row_scale = rs.next_norm = None
+        try:
+            self._sublayer(step, x, self.children["mixer_norm"], lambda xn, y: self.mixer.forward(step, xn, y, cache, owns_cache),
+                           self.children["mixer_out_norm"])
+            if self.ffn is not None:
+                self._sublayer(step, x, self.children["ffn_norm"], lambda xn, y: self.ffn.forward(step, xn, y),
+                               self.children["ffn_out_norm"])
+        finally:
+            rs.overwrite = rs.defer_overwrite = False
+
+
+register_block("sandwich_norm", SandwichNormBlock)

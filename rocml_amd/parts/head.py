@@ -1,7 +1,8 @@
 """The model's output: the norm of the rows whose logits are wanted, then their product with
 the output matrix (rocml/src/forward/chunk_forward.rs:170-184 does both for the last row only).
 A tied output matrix is the embedding's table itself, one buffer
-(rocml/src/weights/mod.rs:48-62 loads it twice)."""
+(rocml/src/weights/mod.rs:48-62 loads it twice).  With a soft cap the logits ``z`` become
+``cap * tanh(z / cap)``."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -22,6 +23,9 @@ class NormLinearHead(Head):
         self.vocab = spec.vocab
         self.hidden = spec.hidden
         self.tied = bool(spec.tied)
+        self.softcap = getattr(spec, "softcap", None)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ConfigError(f"the soft cap of the logits must be positive, got {self.softcap}")
         self.dtype = ctx.dtype
         self.norm = build_norm(spec.norm, ctx)
         self.matrix: Optional[torch.Tensor] = None
@@ -61,6 +65,8 @@ class NormLinearHead(Head):
             self.norm.forward(x, xn, rows=want_rows)
         logits = ws.get("head.logits", (n_want, self.vocab), torch.float32)
         ops.gemm(xn, self.matrix, logits, workspace=ws.scratch())
+        if self.softcap is not None:
+            ops.softcap(logits, self.softcap)
         return logits
 
 

@@ -8,6 +8,9 @@ its columns in the result.  The branches' outputs stay in buffers of their own: 
 that norms after its sum takes them as they are (``branches``) and does the branches' norms, their
 sum, the residual sum and its own norm in one kernel; in any other block ``forward`` adds the
 weighted sum to the stream.
+
+``normed`` false: the branches' outputs are summed as they are (no norms, no gains).  ``branch_weights``: a
+factor per branch instead of one for all.
 """
 from __future__ import annotations
 
@@ -34,6 +37,13 @@ class ParallelMixer(Mixer):
             raise ConfigError(f"the branches of a parallel mixer need different names, got {names}")
         self.spec = spec
         self.dtype = ctx.dtype
+        self.normed = bool(getattr(spec, "normed", True))
+        weights = getattr(spec, "branch_weights", None)
+        if weights is not None and len(weights) != len(spec.branches):
+            raise ConfigError(f"{len(weights)} weights for {len(spec.branches)} branches")
+        self.weights = tuple(float(w) for w in weights) if weights is not None else (float(spec.weight),) * len(spec.branches)
+        if self.normed and len(set(self.weights)) > 1:
+            raise ConfigError("branches that are normed share one weight")
         self.children = {name: build_mixer(sub, ctx) for name, sub in spec.branches}
         self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
         self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
@@ -47,14 +57,15 @@ class ParallelMixer(Mixer):
         for name, child in self.children.items():
             for p, ps in child.param_specs().items():
                 specs[f"{name}.{p}"] = ps
-            specs[f"{name}.out_norm.weight"] = ParamSpec((self.spec.hidden,), role="gain", init="gain")
+            if self.normed:
+                specs[f"{name}.out_norm.weight"] = ParamSpec((self.spec.hidden,), role="gain", init="gain")
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         for name, child in self.children.items():
             prefix = name + "."
             own = {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
-            self.gains[name] = own.pop("out_norm.weight")
+            self.gains[name] = own.pop("out_norm.weight") if self.normed else None
             child.bind(own)
         # One product for all branches that can take its result: their matrices one under the other, each
         # branch's own matrix replaced by its rows of the whole (no second copy stays).
@@ -101,11 +112,14 @@ class ParallelMixer(Mixer):
             ws.flush_pending()
             outs.append(y)
         rs.overwrite, rs.defer_overwrite = before, before_defer
-        return outs, [self.gains[name] for name in self.children], float(self.spec.weight)
+        return outs, [self.gains[name] for name in self.children], self.weights[0]
 
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
         outs, gains, weight = self.branches(step, xn, cache, owns_cache)
         step.workspace.flush_pending()
+        if not self.normed:
+            ops.weighted_sum(x_accum, outs, self.weights, alpha=0.0 if stream(step).overwrite else 1.0)
+            return
         ops.sum_norm(x_accum, outs, gains, None, self.spec.eps, alpha=0.0 if stream(step).overwrite else 1.0, weight=weight)
 
 

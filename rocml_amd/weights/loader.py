@@ -72,11 +72,6 @@ def load_model(path: str, dtype="bfloat16", device="cuda") -> DecoderModel:
     raw = read_config_json(path)
     arch = architecture_of(raw)
     cfg = arch.read_config(raw)
-    spec = arch.to_spec(cfg)
-    model = DecoderModel(spec, compute_dtype(dtype), device=device)
-    model.config = cfg
-    expected = model.param_specs()
-    names = arch.checkpoint_names(spec)
     files = _shard_files(path)
     where: Dict[str, str] = {}
     found: Dict[str, tuple] = {}
@@ -86,6 +81,14 @@ def load_model(path: str, dtype="bfloat16", device="cuda") -> DecoderModel:
                 sl = f.get_slice(name)
                 found[name] = (tuple(sl.get_shape()), sl.get_dtype())
                 where[name] = file
+    if arch.refine_config is not None:
+        # sizes that only the tensors' shapes give
+        cfg = arch.refine_config(cfg, {name: shape for name, (shape, _) in found.items()})
+    spec = arch.to_spec(cfg)
+    model = DecoderModel(spec, compute_dtype(dtype), device=device)
+    model.config = cfg
+    expected = model.param_specs()
+    names = arch.checkpoint_names(spec)
     check_tensors(expected, names, found, unused=arch.unused_tensors(spec))
     tensors: Dict[str, torch.Tensor] = {}
     by_file: Dict[str, List[str]] = {}
