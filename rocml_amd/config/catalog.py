@@ -148,6 +148,45 @@ CATALOG += [
     ModelEntry("sogavik-2b", sogavik_config(32768, 2048, 16, 8, 128, 1024, 16, 128, 32, 1024, 4, 64, 24)),
 ]
 
+
+
+def roravik_config(vocab, width, heads, kv_heads, dim, window, ret_heads, ret_dim, mix_heads, mix_dim, ff, experts, expert_ff, top,
+                   n_layers, loop=None, conv=4, decay_rank=64):
+    """A Roravik configuration: a pair of mixers (a windowed attention whose q, k and v pass a short convolution, with a
+    soft cap and a sink per head, beside a recurrence with a decay per token and channel) in the even layers and a
+    retention in the odd ones; a dense feed-forward and routed experts (two groups of which one is kept, and a shared
+    expert of twice an expert's size) in turn.  ``loop``: ``(start, stop, times)`` or None."""
+    rot = {"base": 10000.0, "dims": dim}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": conv, "scale": dim ** -0.5, "softcap": 30.0,
+            "mask": {"size": window}, "rot": rot}
+    right = {"heads": mix_heads, "dim": mix_dim, "decay_rank": decay_rank}
+    decay = [1.0 - 2.0 ** (-5 - 6 * h / max(ret_heads - 1, 1)) for h in range(ret_heads)]
+    retention = {"heads": ret_heads, "dim": ret_dim, "vdim": ret_dim, "decay": decay, "rot": {"base": 1000000.0, "dims": ret_dim}}
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "groups": {"count": 2, "keep": 1}},
+           "shared": {"ff": 2 * expert_ff}}
+    layers = []
+    for i in range(n_layers):
+        mlp = dense if i % 2 == 0 else moe
+        if i % 2 == 0:
+            layers.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.5, "right_scale": 0.5}, "mlp": mlp})
+        else:
+            layers.append({"type": "retention", "mixer": retention, "mlp": mlp})
+    cfg = {"architecture": "Roravik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": width ** 0.5},
+           "logit_softcap": 30.0, "layers": layers}
+    if loop is not None:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+# The fifth architecture: a test-sized model and the layer sizes of a 2B-class model (random weights; no
+# checkpoint of this design exists).
+CATALOG += [
+    ModelEntry("roravik-tiny", roravik_config(320, 96, 4, 2, 32, 40, 2, 24, 2, 16, 160, 8, 48, 2, 4, loop=(0, 2, 2), decay_rank=8),
+               default_ctx=512, init_norm_jitter=True),
+    ModelEntry("roravik-2b", roravik_config(32768, 2048, 16, 8, 128, 1024, 16, 128, 32, 64, 6144, 32, 1024, 4, 24)),
+]
+
 _BY_NAME = {e.name: e for e in CATALOG}
 
 

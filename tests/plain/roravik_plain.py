@@ -224,3 +224,13 @@ def forward(cfg: Dict, tensors: Dict[str, torch.Tensor], tokens, collect: Option
     z = offset_norm(x, tensors["final.norm"], eps) @ tensors["embed"].T
     cap = float(cfg["logit_softcap"])
     return cap * torch.tanh(z / cap)
+
+
+def greedy(cfg: Dict, tensors: Dict[str, torch.Tensor], prompt, n_new: int) -> List[int]:
+    """``n_new`` tokens, each the largest logit after the prompt and the tokens before it."""
+    tokens = list(prompt)
+    out = []
+    for _ in range(n_new):
+        out.append(int(forward(cfg, tensors, tokens)[-1].argmax()))
+        tokens.append(out[-1])
+    return out
