@@ -52,6 +52,53 @@ def short_conv(u: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def recurrence_read_after(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay) -> torch.Tensor:
+    """``q, k [T, H, d]``, ``v [T, H, dv]``, one decay per head: ``S_t = decay S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t``."""
+    T, H, d = q.shape
+    out = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for a in range(H):
+        S = torch.zeros(d, v.shape[-1], dtype=q.dtype)
+        for t in range(T):
+            S = float(decay[a]) * S + torch.outer(k[t, a], v[t, a])
+            out[t, a] = S.T @ q[t, a]
+    return out
+
+
+def recurrence_read_before(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    """``r, k, w [T, H, d]``, ``v [T, H, dv]``, ``u [H, d]``: ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t``, then
+    ``S_t = diag(w_t) S_(t-1) + k_t v_t^T``."""
+    T, H, d = r.shape
+    out = torch.zeros(T, H, v.shape[-1], dtype=r.dtype)
+    for a in range(H):
+        S = torch.zeros(d, v.shape[-1], dtype=r.dtype)
+        for t in range(T):
+            kv = torch.outer(k[t, a], v[t, a])
+            out[t, a] = (S + u[a][:, None] * kv).T @ r[t, a]
+            S = w[t, a][:, None] * S + kv
+    return out
+
+
+def capped_window_softmax(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, cap: float, window: int,
+                          sink: torch.Tensor) -> torch.Tensor:
+    """``q [T, H, d]``, ``k [T, G, d]``, ``v [T, G, dv]`` of one sequence: ``s = cap tanh(scale (q . k) / cap)``, position
+    ``i`` sees ``j`` with ``0 <= i - j < window``, and the denominator has one more term ``exp(sink_a)``."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    pos = torch.arange(T)
+    dist = pos[:, None] - pos[None, :]
+    seen = (dist >= 0) & (dist < window)
+    out = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for a in range(H):
+        g = a // (H // G)
+        s = (q[:, a] @ k[:, g].T) * scale
+        s = cap * torch.tanh(s / cap)
+        s = s.masked_fill(~seen, float("-inf"))
+        top = torch.maximum(s.max(dim=-1, keepdim=True).values, sink[a])
+        e = torch.exp(s - top)
+        out[:, a] = (e @ v[:, g]) / (e.sum(dim=-1, keepdim=True) + torch.exp(sink[a] - top))
+    return out
+
+
 def retention(h: torch.Tensor, p: Dict[str, torch.Tensor], m: Dict, eps: float) -> torch.Tensor:
     """Linear attention with one fixed decay per head, no softmax and no denominator: per head
     ``S_t = decay S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t``; q and k rotated, k times ``dim^(-1/2)``
@@ -63,12 +110,7 @@ def retention(h: torch.Tensor, p: Dict[str, torch.Tensor], m: Dict, eps: float) 
     q = rotate((h @ p["q"].T).view(T, H, d), pos, m["rot"])
     k = rotate((h @ p["k"].T).view(T, H, d), pos, m["rot"]) * d ** -0.5
     v = (h @ p["v"].T).view(T, H, dv)
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
-    for a in range(H):
-        S = torch.zeros(d, dv, dtype=h.dtype)
-        for t in range(T):
-            S = m["decay"][a] * S + torch.outer(k[t, a], v[t, a])
-            out[t, a] = S.T @ q[t, a]
+    out = recurrence_read_after(q, k, v, m["decay"])
     out = rms(out, eps).reshape(T, H * dv) * silu(h @ p["g"].T)
     return out @ p["o"].T
 
@@ -84,18 +126,7 @@ def window_attention(h: torch.Tensor, p: Dict[str, torch.Tensor], m: Dict) -> to
     k = short_conv(h @ p["k"].T, p["k.conv"]).view(T, G, d)
     v = short_conv(h @ p["v"].T, p["v.conv"]).view(T, G, dv)
     q, k = rotate(q, pos, m["rot"]), rotate(k, pos, m["rot"])
-    cap, window = float(m["softcap"]), m["mask"]["size"]
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
-    dist = pos[:, None] - pos[None, :]
-    seen = (dist >= 0) & (dist < window)
-    for a in range(H):
-        g = a // (H // G)
-        s = (q[:, a] @ k[:, g].T) * float(m["scale"])
-        s = cap * torch.tanh(s / cap)
-        s = s.masked_fill(~seen, float("-inf"))
-        top = torch.maximum(s.max(dim=-1, keepdim=True).values, p["sink"][a])
-        e = torch.exp(s - top)
-        out[:, a] = (e @ v[:, g]) / (e.sum(dim=-1, keepdim=True) + torch.exp(p["sink"][a] - top))
+    out = capped_window_softmax(q, k, v, float(m["scale"]), float(m["softcap"]), m["mask"]["size"], p["sink"])
     return out.reshape(T, H * dv) @ p["o"].T
 
 
@@ -116,13 +147,7 @@ def time_mix(h: torch.Tensor, p: Dict[str, torch.Tensor], m: Dict, eps: float) -
     v = (mix("v") @ p["v"].T).view(T, H, d)
     gate = silu(mix("g") @ p["g"].T)
     w = torch.exp(-torch.exp(torch.tanh(mix("w") @ p["w1"].T) @ p["w2"].T + p["w0"][None, :])).view(T, H, d)
-    out = torch.zeros(T, H, d, dtype=h.dtype)
-    for a in range(H):
-        S = torch.zeros(d, d, dtype=h.dtype)
-        for t in range(T):
-            kv = torch.outer(k[t, a], v[t, a])
-            out[t, a] = (S + p["u"][a][:, None] * kv).T @ r[t, a]
-            S = w[t, a][:, None] * S + kv
+    out = recurrence_read_before(r, k, v, w, p["u"])
     out = rms(out, eps).reshape(T, H * d) * p["norm"][None, :] * gate
     return out @ p["o"].T
 
