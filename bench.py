@@ -2,7 +2,7 @@
 """Decode and prefill speed of the Qwen3 shapes with random bfloat16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-8b|qwen3-14b|qwen3-32b]
-    python bench.py --design dokulix|felovik|sogavik [--design-size 2b|8b|14b] [--layers N]
+    python bench.py --design dokulix|felovik|sogavik|roravik [--design-size 2b|8b|14b] [--layers N]
 
 The default run is the Qwen3-8B shape.  A step is one decode step of a batch of 8 sequences,
 each with a 2,048-token random prompt in the cache (context length 4,096): the engine's step
@@ -33,6 +33,11 @@ in turn, four of 32 experts a token, as many active feed-forward weights as the 
 a windowed attention beside a matrix memory; routed experts and a token-side input in every layer, norms on the
 sublayers' outputs) beside the Felovik model of the same sizes, the library's closest design (a pair of mixers
 with a recurrence, routed experts).
+``--design roravik`` measures a Roravik model (a windowed attention with convolved q, k and v, a soft cap and a sink per
+head beside a recurrence with a decay per token and channel in the even layers, a retention in the odd ones; dense
+feed-forwards and routed experts with a shared expert in turn; a norm before and after every sublayer) beside the
+Felovik model of the same sizes, the library's closest design (a pair of mixers with a recurrence in every layer,
+dense feed-forwards and routed experts in turn).
 
 The workloads follow the reference's bench (rocml-cli/src/cmd_bench.rs:79-243): synthetic
 prompts, greedy, no stop token, warm-up first; times are taken around synchronised steps.
@@ -78,7 +83,7 @@ def felovik_config(z: dict, n_layers: int):
             "layers": [{"type": "parallel", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe} for i in range(n_layers)]}
 
 
-COMPANION = {"dokulix": "qwen3", "felovik": "qwen3", "sogavik": "felovik"}     # the closest model each design is measured beside
+COMPANION = {"dokulix": "qwen3", "felovik": "qwen3", "sogavik": "felovik", "roravik": "felovik"}     # the closest model each design is measured beside
 
 
 def design_configs(size: dict, n_layers: int, design: str = "dokulix"):
@@ -88,6 +93,12 @@ def design_configs(size: dict, n_layers: int, design: str = "dokulix"):
         from rocml_amd.config.catalog import sogavik_config
         return (sogavik_config(z["vocab"], z["width"], z["heads"], z["kv_heads"], z["dim"], z["window"], z["width"] // 128, 128,
                                32, z["ff"] // 4, 4, 64, n_layers, parallel_every=2), felovik_config(z, n_layers))
+    if design == "roravik":
+        from rocml_amd.config.catalog import roravik_config
+        # recurrence heads of 64 with an inner width equal to the model's, retention heads of 128 likewise, experts as the
+        # companion's (32 of a quarter of the dense size, 4 a token)
+        return (roravik_config(z["vocab"], z["width"], z["heads"], z["kv_heads"], z["dim"], z["window"], z["width"] // 128, 128,
+                               z["width"] // 64, 64, z["ff"], 32, z["ff"] // 4, 4, n_layers), felovik_config(z, n_layers))
     att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
            "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
                      "mask": {"size": z["chunk"]}, "scale": z["dim"] ** -0.5}}
@@ -195,7 +206,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points")
     ap.add_argument("--prefill-runs", type=int, default=3)
-    ap.add_argument("--design", default=None, choices=["dokulix", "felovik", "sogavik"],
+    ap.add_argument("--design", default=None, choices=["dokulix", "felovik", "sogavik", "roravik"],
                     help="measure this architecture at real layer sizes beside the closest Qwen3 shape, instead of the default workload")
     ap.add_argument("--design-size", default="2b", choices=sorted(DESIGN_SIZES), help="layer sizes for --design")
     ap.add_argument("--skip-prompts", action="store_true",

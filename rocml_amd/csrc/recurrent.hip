@@ -1108,18 +1108,25 @@ ROCML_EXPORT int rocml_gated_part_norm(const float* y, const float* z, int ldz, 
 //   after the update (a retention):        o_t = S_t^T q_t, with w_t one constant per head;
 //   before it, with a bonus on the token:  o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t, with w_t per token and channel.
 // The columns of S (one per value) do not depend on each other: a block takes (sequence, head, 16 values), the 16
-// lanes of a row of lanes hold one column, lane l the entries l, l + 16, ..., and add their parts of the dot product
-// with q across the row.  Four tokens are worked on at a time (all their operands are requested first).  The state
+// lanes of a row of lanes hold one column, lane l the R entries l R .. l R + R - 1, and add their parts of the dot
+// product with q across the row.  The tokens' rows (q, k, the decays and the block's 16 values) come in chunks of 16
+// tokens through LDS: every thread owns up to DS_SLOTS columns of a chunk's rows, requests the next chunk's numbers
+// into registers before it works on this one, and writes them to LDS when this one is done, so the walk over the
+// tokens waits for memory once.  Inside a chunk four tokens are worked on at a time (their cross-lane sums side by
+// side).  w_logit: the decays come as logits x and are exp(-exp(x + offset)), formed on the way into LDS.  The state
 // is stored column by column, [slot, head, dv, dk].  Everything is 32-bit.
 constexpr int DS_COLS = 16;      // values (columns of the state) per block
 constexpr int DS_LANES = 16;     // lanes that share a column
-constexpr int DS_TOKENS = 4;     // tokens in flight
+constexpr int DS_THREADS = DS_COLS * DS_LANES;
+constexpr int DS_CHUNK = 16;     // tokens of a chunk
+constexpr int DS_TOKENS = 4;     // tokens whose sums cross the lanes together
 
 struct DecayScanArgs {
     const float* q; int ldq; int q_col0;
     const float* k; int ldk; int k_col0;
     const float* v; int ldv; int v_col0;
     const float* w; int ldw; int w_col0;      // per token and channel, or null
+    const float* w_offset;                     // [H * dk] or null: w holds logits x, the decay is exp(-exp(x + offset))
     const float* head_decay;                   // [H], or null (then w)
     const float* bonus;                        // [H * dk], or null: the state is read after its update
     float* state; const int* cu_seqlens; const int* seq_slots;
@@ -1134,73 +1141,121 @@ __device__ __forceinline__ float ds_row_sum(float v) {
     return v;
 }
 
-template <int R, bool BONUS>
-__global__ void __launch_bounds__(DS_COLS * DS_LANES)
+// R: entries of a column per lane (dk <= 16 R).  PER_TOKEN: a decay per token and channel (else one per head).
+template <int R, bool BONUS, bool PER_TOKEN>
+__global__ void __launch_bounds__(DS_THREADS)
 decay_scan_kernel(DecayScanArgs a) {
+    constexpr int ARRAYS = PER_TOKEN ? 3 : 2;                       // q, k (and the decays), each dk wide, then 16 values
+    constexpr int MAX_ROW = ARRAYS * 16 * R + DS_COLS;
+    constexpr int DS_SLOTS = (MAX_ROW + DS_THREADS - 1) / DS_THREADS;
+    extern __shared__ float ds_rows[];                               // [DS_CHUNK][row]
     int b = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
-    int l = threadIdx.x % DS_LANES, c = threadIdx.x / DS_LANES;
+    int tid = threadIdx.x;
+    int l = tid % DS_LANES, c = tid / DS_LANES;
+    int dk = a.dk;
+    int row = ARRAYS * dk + DS_COLS;
     int col = tile * DS_COLS + c;
     bool col_ok = col < a.dv;
     int first = a.cu_seqlens[b], n = a.cu_seqlens[b + 1] - first;
-    float* st = a.state + (((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv + (col_ok ? col : 0)) * a.dk;
+    // the columns of a chunk's rows that this thread brings in: where they come from, per slot
+    const float* src[DS_SLOTS];
+    int src_ld[DS_SLOTS];
+    float offset[DS_SLOTS];
+    bool is_logit[DS_SLOTS];
+#pragma unroll
+    for (int m = 0; m < DS_SLOTS; ++m) {
+        int x = tid + m * DS_THREADS;
+        src[m] = nullptr;
+        src_ld[m] = 0;
+        offset[m] = 0.f;
+        is_logit[m] = false;
+        if (x < dk) { src[m] = a.q + a.q_col0 + (size_t)h * dk + x; src_ld[m] = a.ldq; }
+        else if (x < 2 * dk) { src[m] = a.k + a.k_col0 + (size_t)h * dk + (x - dk); src_ld[m] = a.ldk; }
+        else if (PER_TOKEN && x < 3 * dk) {
+            src[m] = a.w + a.w_col0 + (size_t)h * dk + (x - 2 * dk);
+            src_ld[m] = a.ldw;
+            if (a.w_offset) { is_logit[m] = true; offset[m] = a.w_offset[(size_t)h * dk + (x - 2 * dk)]; }
+        } else if (x < row) {
+            int vc = tile * DS_COLS + (x - ARRAYS * dk);
+            if (vc < a.dv) { src[m] = a.v + a.v_col0 + (size_t)h * a.dv + vc; src_ld[m] = a.ldv; }
+        }
+    }
+    float* st = a.state + (((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv + (col_ok ? col : 0)) * dk;
     float s[R], u[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        int i = l + r * DS_LANES;
-        s[r] = (col_ok && i < a.dk) ? st[i] : 0.f;
-        u[r] = (BONUS && i < a.dk) ? a.bonus[(size_t)h * a.dk + i] : 0.f;
+        int i = l * R + r;
+        s[r] = (col_ok && i < dk) ? st[i] : 0.f;
+        u[r] = (BONUS && i < dk) ? a.bonus[(size_t)h * dk + i] : 0.f;
     }
-    float hd = a.head_decay ? a.head_decay[h] : 0.f;
-    for (int t0 = 0; t0 < n; t0 += DS_TOKENS) {
-        float q[DS_TOKENS][R], k[DS_TOKENS][R], w[DS_TOKENS][R], v[DS_TOKENS];
+    float hd = PER_TOKEN ? 0.f : a.head_decay[h];
+    float next[DS_SLOTS][DS_CHUNK];
+    auto request = [&](int t0) {
 #pragma unroll
-        for (int j = 0; j < DS_TOKENS; ++j) {
-            bool ok = t0 + j < n;
-            size_t row = (size_t)(first + (ok ? t0 + j : 0));
-            v[j] = (ok && col_ok) ? a.v[row * a.ldv + a.v_col0 + (size_t)h * a.dv + col] : 0.f;
+        for (int m = 0; m < DS_SLOTS; ++m)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                int i = l + r * DS_LANES;
-                bool in = ok && i < a.dk;
-                size_t e = (size_t)h * a.dk + i;
-                q[j][r] = in ? a.q[row * a.ldq + a.q_col0 + e] : 0.f;
-                k[j][r] = in ? a.k[row * a.ldk + a.k_col0 + e] : 0.f;
-                w[j][r] = a.w ? (in ? a.w[row * a.ldw + a.w_col0 + e] : 1.f) : hd;
-            }
-        }
-        float acc[DS_TOKENS];
+            for (int j = 0; j < DS_CHUNK; ++j)
+                next[m][j] = (src[m] && t0 + j < n) ? src[m][(size_t)(first + t0 + j) * src_ld[m]] : 0.f;
+    };
+    request(0);
+    for (int t0 = 0; t0 < n; t0 += DS_CHUNK) {
 #pragma unroll
-        for (int j = 0; j < DS_TOKENS; ++j) {
-            float sum = 0.f;
-            if (t0 + j < n) {
+        for (int m = 0; m < DS_SLOTS; ++m) {
+            int x = tid + m * DS_THREADS;
+            if (x < row) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    float kv = k[j][r] * v[j];
-                    if constexpr (BONUS) {
-                        sum = fmaf(fmaf(u[r], kv, s[r]), q[j][r], sum);
-                        s[r] = fmaf(w[j][r], s[r], kv);
-                    } else {
-                        s[r] = fmaf(w[j][r], s[r], kv);
-                        sum = fmaf(s[r], q[j][r], sum);
-                    }
+                for (int j = 0; j < DS_CHUNK; ++j) {
+                    float val = next[m][j];
+                    if (PER_TOKEN && is_logit[m]) val = expf(-expf(val + offset[m]));
+                    ds_rows[j * row + x] = val;
                 }
             }
-            acc[j] = sum;
         }
+        __syncthreads();
+        if (t0 + DS_CHUNK < n) request(t0 + DS_CHUNK);
+        int here = min(DS_CHUNK, n - t0);
+        for (int j0 = 0; j0 < here; j0 += DS_TOKENS) {
+            float acc[DS_TOKENS];
 #pragma unroll
-        for (int j = 0; j < DS_TOKENS; ++j) acc[j] = ds_row_sum(acc[j]);
-        if (l < DS_TOKENS && col_ok) {
-            float mine = acc[0];
+            for (int jj = 0; jj < DS_TOKENS; ++jj) {
+                const float* tok = ds_rows + (j0 + jj) * row;
+                float sum = 0.f;
+                if (j0 + jj < here) {
+                    float vv = tok[ARRAYS * dk + c];
 #pragma unroll
-            for (int j = 1; j < DS_TOKENS; ++j) mine = l == j ? acc[j] : mine;
-            if (t0 + l < n) a.out[(size_t)(first + t0 + l) * a.n_heads * a.dv + (size_t)h * a.dv + col] = mine;
+                    for (int r = 0; r < R; ++r) {
+                        int i = l * R + r;
+                        bool in = i < dk;
+                        float qq = in ? tok[i] : 0.f;
+                        float kv = (in ? tok[dk + i] : 0.f) * vv;
+                        float ww = PER_TOKEN ? (in ? tok[2 * dk + i] : 0.f) : hd;
+                        if constexpr (BONUS) {
+                            sum = fmaf(fmaf(u[r], kv, s[r]), qq, sum);
+                            s[r] = fmaf(ww, s[r], kv);
+                        } else {
+                            s[r] = fmaf(ww, s[r], kv);
+                            sum = fmaf(s[r], qq, sum);
+                        }
+                    }
+                }
+                acc[jj] = sum;
+            }
+#pragma unroll
+            for (int jj = 0; jj < DS_TOKENS; ++jj) acc[jj] = ds_row_sum(acc[jj]);
+            if (l < DS_TOKENS && col_ok) {
+                float mine = acc[0];
+#pragma unroll
+                for (int jj = 1; jj < DS_TOKENS; ++jj) mine = l == jj ? acc[jj] : mine;
+                if (j0 + l < here) a.out[(size_t)(first + t0 + j0 + l) * a.n_heads * a.dv + (size_t)h * a.dv + col] = mine;
+            }
         }
+        __syncthreads();                         // the rows are rewritten by the next chunk
     }
     if (col_ok) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            int i = l + r * DS_LANES;
-            if (i < a.dk) st[i] = s[r];
+            int i = l * R + r;
+            if (i < dk) st[i] = s[r];
         }
     }
 }
@@ -1208,25 +1263,30 @@ decay_scan_kernel(DecayScanArgs a) {
 template <int R>
 static void launch_decay_scan(const DecayScanArgs& a, int n_seqs, hipStream_t stream) {
     dim3 grid(n_seqs, a.n_heads, ceil_div(a.dv, DS_COLS));
-    if (a.bonus) decay_scan_kernel<R, true><<<grid, DS_COLS * DS_LANES, 0, stream>>>(a);
-    else decay_scan_kernel<R, false><<<grid, DS_COLS * DS_LANES, 0, stream>>>(a);
+    size_t lds = (size_t)DS_CHUNK * ((a.w ? 3 : 2) * a.dk + DS_COLS) * sizeof(float);
+    if (a.w && a.bonus) decay_scan_kernel<R, true, true><<<grid, DS_THREADS, lds, stream>>>(a);
+    else if (a.w) decay_scan_kernel<R, false, true><<<grid, DS_THREADS, lds, stream>>>(a);
+    else if (a.bonus) decay_scan_kernel<R, true, false><<<grid, DS_THREADS, lds, stream>>>(a);
+    else decay_scan_kernel<R, false, false><<<grid, DS_THREADS, lds, stream>>>(a);
 }
 
 ROCML_EXPORT int rocml_decay_scan(const float* q, int ldq, int q_col0, const float* k, int ldk, int k_col0, const float* v,
-                                  int ldv, int v_col0, const float* w, int ldw, int w_col0, const float* head_decay,
-                                  const float* bonus, float* state, int n_slots, const int* cu_seqlens, const int* seq_slots,
-                                  int n_seqs, int n_tokens, float* out, int n_heads, int dk, int dv, hipStream_t stream) {
+                                  int ldv, int v_col0, const float* w, int ldw, int w_col0, const float* w_offset,
+                                  const float* head_decay, const float* bonus, float* state, int n_slots, const int* cu_seqlens,
+                                  const int* seq_slots, int n_seqs, int n_tokens, float* out, int n_heads, int dk, int dv,
+                                  hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && n_slots > 0 && n_heads > 0 && dk > 0 && dv > 0, "decay_scan: bad sizes T=%d B=%d H=%d",
                   n_tokens, n_seqs, n_heads);
     ROCML_REQUIRE(dk <= 16 * DS_LANES, "decay_scan: a key size of %d exceeds %d", dk, 16 * DS_LANES);
     ROCML_REQUIRE(q && k && v && state && cu_seqlens && seq_slots && out, "decay_scan: missing arguments");
     ROCML_REQUIRE((w != nullptr) != (head_decay != nullptr), "decay_scan: a decay per token and channel or one per head, one of the two");
+    ROCML_REQUIRE(!w_offset || w, "decay_scan: an offset goes with decays given as logits");
     ROCML_REQUIRE(q_col0 >= 0 && k_col0 >= 0 && v_col0 >= 0 && ldq >= q_col0 + n_heads * dk && ldk >= k_col0 + n_heads * dk &&
                       ldv >= v_col0 + n_heads * dv && (!w || (w_col0 >= 0 && ldw >= w_col0 + n_heads * dk)),
                   "decay_scan: a row stride is too small for its columns");
     if (n_tokens == 0 || n_seqs == 0) return 0;
-    DecayScanArgs a{q, ldq, q_col0, k, ldk, k_col0, v, ldv, v_col0, w, ldw, w_col0, head_decay, bonus, state, cu_seqlens, seq_slots,
-                    out, n_heads, dk, dv};
+    DecayScanArgs a{q, ldq, q_col0, k, ldk, k_col0, v, ldv, v_col0, w, ldw, w_col0, w_offset, head_decay, bonus, state, cu_seqlens,
+                    seq_slots, out, n_heads, dk, dv};
     int r = ceil_div(dk, DS_LANES);
     if (r <= 1) launch_decay_scan<1>(a, n_seqs, stream);
     else if (r <= 2) launch_decay_scan<2>(a, n_seqs, stream);

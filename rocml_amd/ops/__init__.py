@@ -60,7 +60,7 @@ _SIGNATURES = {
         "rocml_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _F, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
         "rocml_mlstm_tile": [],
         "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
-        "rocml_decay_scan": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
+        "rocml_decay_scan": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
         "rocml_rotate_rows": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P],
         "rocml_shift_mix": [_P, _I, _I, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P],
         "rocml_tanh": [_P, _P, _I, _LL, _P],
@@ -1247,14 +1247,16 @@ def head_norm_gate(o: torch.Tensor, g: torch.Tensor, g_col0: int, gain: Optional
 def decay_scan(q: torch.Tensor, q_col0: int, k: torch.Tensor, k_col0: int, v: torch.Tensor, v_col0: int,
                state: torch.Tensor, cu_seqlens: torch.Tensor, seq_slots: torch.Tensor, out: torch.Tensor,
                n_heads: int, head_dim: int, v_head_dim: int, head_decay: Optional[torch.Tensor] = None,
-               decay: Optional[torch.Tensor] = None, decay_col0: int = 0, bonus: Optional[torch.Tensor] = None) -> None:
+               decay: Optional[torch.Tensor] = None, decay_col0: int = 0, bonus: Optional[torch.Tensor] = None,
+               decay_offset: Optional[torch.Tensor] = None) -> None:
     """A recurrence whose state per head, ``S [dk, dv]``, decays row by row, over the step's tokens, per sequence in
     order: ``S <- diag(w_t) S + k_t v_t^T``.  With ``head_decay`` (one number per head) ``w_t`` is that constant and
     the output reads the new state, ``o_t = S_t^T q_t``; with ``decay`` (per token and key channel, columns
     ``decay_col0 ..`` of a 32-bit matrix) and ``bonus`` ``u [H * dk]`` the output reads the state before the update,
-    ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t``.  q, k, v are column ranges of 32-bit matrices ``[T, ld]``;
+    ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t``.  With ``decay_offset`` (``[H * dk]``) ``decay`` holds logits ``x`` and the
+    decay is ``exp(-exp(x + decay_offset))``.  q, k, v are column ranges of 32-bit matrices ``[T, ld]``;
     ``state [slots, H, dv, dk]``; ``out [T, H * dv]``; all 32-bit."""
-    _dev(q, k, v, state, cu_seqlens, seq_slots, out, head_decay, decay, bonus)
+    _dev(q, k, v, state, cu_seqlens, seq_slots, out, head_decay, decay, bonus, decay_offset)
     for t, what in ((q, "queries"), (k, "keys"), (v, "values"), (state, "recurrent state"), (out, "recurrence output")):
         _want(t, torch.float32, what)
     n_tokens, n_seqs = out.shape[0], seq_slots.numel()
@@ -1265,14 +1267,18 @@ def decay_scan(q: torch.Tensor, q_col0: int, k: torch.Tensor, k_col0: int, v: to
         raise KernelError("recurrence inputs, output or tables do not fit the step")
     if (head_decay is None) == (decay is None) or (decay is None) != (bonus is None):
         raise KernelError("the recurrence takes one decay per head, or a decay per token and channel together with a bonus")
-    for t, n, what in ((head_decay, n_heads, "the heads' decays"), (bonus, n_heads * head_dim, "the bonus")):
+    if decay_offset is not None and decay is None:
+        raise KernelError("an offset of the decays' logits goes with decays per token")
+    for t, n, what in ((head_decay, n_heads, "the heads' decays"), (bonus, n_heads * head_dim, "the bonus"),
+                       (decay_offset, n_heads * head_dim, "the offset of the decays' logits")):
         if t is not None and (t.dtype != torch.float32 or t.numel() != n):
             raise KernelError(f"{what} must be 32-bit with {n} numbers")
     if decay is not None and (decay.dtype != torch.float32 or decay.dim() != 2 or decay.shape[0] != n_tokens):
         raise KernelError("the decays per token must be a 32-bit matrix with a row per token")
     _check("recurrent", library("recurrent").rocml_decay_scan(
         _ptr(q), q.shape[1], q_col0, _ptr(k), k.shape[1], k_col0, _ptr(v), v.shape[1], v_col0, _ptr(decay),
-        0 if decay is None else decay.shape[1], decay_col0, _ptr(head_decay), _ptr(bonus), _ptr(state), state.shape[0],
+        0 if decay is None else decay.shape[1], decay_col0, _ptr(decay_offset), _ptr(head_decay), _ptr(bonus), _ptr(state),
+        state.shape[0],
         _ptr(cu_seqlens), _ptr(seq_slots), n_seqs, n_tokens, _ptr(out), n_heads, head_dim, v_head_dim, _stream()))
 
 

@@ -3,8 +3,8 @@
 With ``h'`` the previous token's input (the sequence's kept row; zeros before its first token), each of r, k, v, the
 gate and the decay reads a mix of its own, ``h + (h' - h) mu``, formed in 32-bit and rounded to the compute type for
 the products.  ``r``, ``k``, ``v`` and the gate come from four products into one 32-bit buffer; the decay is
-``w = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0))`` (two small products with ``tanh`` between them, the offset and both
-exponentials in 32-bit).  Per head, in 32-bit, ``o = (S + diag(u) k v^T)^T r`` and then ``S <- diag(w) S + k v^T``.
+``w = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0))`` (two small products with ``tanh`` between them; the offset and both
+exponentials in 32-bit, inside the recurrence kernel).  Per head, in 32-bit, ``o = (S + diag(u) k v^T)^T r`` and then ``S <- diag(w) S + k v^T``.
 Every head's output is divided by its root mean square, the heads side by side are multiplied by a gain and by
 ``silu(gate)``, rounded to the compute type and projected back.  The cache holds two things per sequence, both zero
 at its start: ``S`` (stored column by column, ``[heads, head_dim, head_dim]``) and the previous token's input.  A
@@ -94,10 +94,10 @@ class TimeMix(Mixer):
         ops.tanh(low, low_act)
         decay = ws.get("timemix.decay", (n, self.inner), torch.float32)
         ops.gemm(low_act, self.w2, decay, workspace=ws.scratch())
-        ops.double_exp_decay(decay, self.w0)
         o = ws.get("timemix.o", (n, self.inner), torch.float32)
+        # (the recurrence kernel turns the logits into decays, exp(-exp(x + w0)), on their way into its LDS)
         ops.decay_scan(proj, 0, proj, self.inner, proj, 2 * self.inner, state.state, step.cu_seqlens, step.seq_slots, o,
-                       s.n_heads, s.head_dim, s.head_dim, decay=decay, decay_col0=0, bonus=self.bonus)
+                       s.n_heads, s.head_dim, s.head_dim, decay=decay, decay_col0=0, bonus=self.bonus, decay_offset=self.w0)
         gated = ws.get("timemix.gated", (n, self.inner), self.dtype)
         ops.head_norm_gate(o, proj, 3 * self.inner, self.norm_gain, gated, s.n_heads, s.eps, gate="silu")
         stream(step).add_product(gated, self.w_out, x_accum)

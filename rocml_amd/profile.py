@@ -103,7 +103,8 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "gemm_residual_prescale": ("product", lambda x, w, resid, gain, xg, ssq, *a, **kw: (
         _nbytes(x, w, resid, resid, gain, xg, ssq), 2 * x.shape[0] * w.shape[0] * x.shape[1])),
     "attention": (lambda *a, **kw: "attention over latent rows" if kw.get("values_in_keys") else
-                  "attention (blocks, slopes, sink)" if kw.get("chunk") or kw.get("sink") or kw.get("slopes") is not None
+                  "attention (blocks, slopes, sink, soft cap)" if kw.get("chunk") or kw.get("sink") or kw.get("slopes") is not None
+                  or kw.get("softcap") is not None
                   else "attention", _attention_cost),
     "attention_decode_fused": ("attention (norm, rotation, append)", _fused_attention_cost),
     "attention_prefill_fused": ("attention (query norm, rotation)", _prefill_fused_cost),
@@ -137,7 +138,7 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
                        proj.shape[0] * n_heads * (2 * head_dim + v_head_dim + 2) * 4 + _nbytes(out)
                        + 2 * slots.numel() * n_heads * head_dim * (v_head_dim + 1) * 4,
                        4 * proj.shape[0] * n_heads * head_dim * (v_head_dim + 1), PEAK_FLOPS[torch.float32])),
-    "head_norm_gate": ("head norm and gate", lambda o, g, g_col0, gain, out, n_heads, eps: (
+    "head_norm_gate": ("head norm and gate", lambda o, g, g_col0, gain, out, n_heads, eps, **kw: (
         2 * _nbytes(o) + _nbytes(out), 8 * o.numel())),
     "splitk_reduce": ("sum of K pieces", _tensor_args_cost()),
     "sum_norm": ("residual sum and norm", lambda x, branches, gains, gain, eps, **kw: (
@@ -158,6 +159,21 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
         + out.shape[0] * (w.shape[2] * a.element_size() + w.shape[1] * out.element_size()),
         2 * out.shape[0] * w.shape[1] * w.shape[2] * (2 if w2 is not None else 1))),
     "moe_combine": ("weighted sum of experts", lambda y, plan, weight, out, **kw: (_nbytes(y, out), 2 * y.numel())),
+    "decay_scan": ("recurrence with a decay per channel (32-bit vector work)",
+                   lambda q, q0, k, k0, v, v0, state, cu, slots, out, n_heads, head_dim, v_head_dim, **kw: (
+                       out.shape[0] * n_heads * ((3 if kw.get("decay") is not None else 2) * head_dim + v_head_dim) * 4 + _nbytes(out)
+                       + 2 * slots.numel() * n_heads * head_dim * v_head_dim * 4,
+                       (6 if kw.get("bonus") is not None else 4) * out.shape[0] * n_heads * head_dim * v_head_dim,
+                       PEAK_FLOPS[torch.float32])),
+    "rotate_rows": ("rotation inside the projection", lambda buf, col0, n_heads, head_dim, rot_dim, cos, sin, scale=1.0: (
+        2 * buf.shape[0] * n_heads * head_dim * 4 + _nbytes(cos, sin), 3 * buf.shape[0] * n_heads * head_dim)),
+    "shift_mix": ("mixes with the previous token", lambda h, mu, state, token_seq, cu, slots, out: (_nbytes(h, mu, out), 2 * out.numel())),
+    "tanh": ("tanh between the decay's matrices", lambda x, out: (_nbytes(x, out), 10 * x.numel())),
+    "double_exp_decay": ("decay from its logits", lambda x, offset: (2 * _nbytes(x), 20 * x.numel())),
+    "softcap": ("soft cap of the logits", lambda x, cap: (2 * _nbytes(x), 10 * x.numel())),
+    "weighted_sum": ("weighted sum of branches", lambda out, branches, weights, alpha=0.0: (
+        _nbytes(out, *branches) + (_nbytes(out) if alpha else 0), 2 * out.numel() * len(branches))),
+    "row_gate_add": ("gated row sum", lambda x, y, gate: (2 * _nbytes(x) + _nbytes(y), 2 * x.numel())),
     "argmax": ("argmax", _tensor_args_cost()),
     "sample": ("sampling", lambda logits, *a, **kw: (_nbytes(logits), 0)),
 }

@@ -46,8 +46,8 @@ def _pieces(lengths, cuts):
 
 
 @pytest.mark.parametrize("dk,dv", [(1, 12), (6, 1), (17, 9), (20, 36), (64, 64), (128, 32), (256, 16)])
-@pytest.mark.parametrize("bonus", [False, True])
-def test_recurrences_through_pieces_and_slots(dk, dv, bonus):
+@pytest.mark.parametrize("bonus,logits", [(False, False), (True, False), (True, True)])
+def test_recurrences_through_pieces_and_slots(dk, dv, bonus, logits):
     """Three sequences of unequal length in slots of their own beside slots of others, brought in pieces of 1 to 40
     tokens; a head that forgets nothing and one that keeps nothing."""
     from rocml_amd import ops
@@ -62,6 +62,7 @@ def test_recurrences_through_pieces_and_slots(dk, dv, bonus):
         w[:, 0] = 1.0
         w[:, 1] = 0.0
         u = torch.randn(H, dk, generator=g, dtype=D64)
+        offset = torch.randn(H, dk, generator=g, dtype=D64)
         want = torch.cat([plain.recurrence_read_before(q[s:s + n], k[s:s + n], v[s:s + n], w[s:s + n], u) for s, n in zip(starts, lengths)])
     else:
         decay = [1.0, 0.0, 0.93]
@@ -81,10 +82,15 @@ def test_recurrences_through_pieces_and_slots(dk, dv, bonus):
         out = torch.empty(len(rows), H * dv, dtype=torch.float32, device=DEV)
         kw = dict(decay=w[rows].reshape(len(rows), -1).float().to(DEV).contiguous(), bonus=u.reshape(-1).float().to(DEV)) if bonus \
             else dict(head_decay=torch.tensor(decay, dtype=torch.float32, device=DEV))
+        if bonus and logits:
+            # the decays as logits x with an offset: w = exp(-exp(x + offset)); the heads that forget nothing and everything
+            # get logits far below and far above zero
+            x = torch.log(-torch.log(w[rows].clamp(1e-30, 1 - 1e-12))).clamp(-40.0, 40.0) - offset
+            kw.update(decay=x.reshape(len(rows), -1).float().to(DEV).contiguous(), decay_offset=offset.reshape(-1).float().to(DEV))
         ops.decay_scan(mat, 3, mat, 3 + H * dk, mat, 3 + 2 * H * dk, state, _i32(cu), _i32([slots[b] for b, _, _ in step]), out,
                        H, dk, dv, **kw)
         got[rows] = out.cpu()
-    _close(got, want.reshape(T, -1), 2e-5, "recurrence")
+    _close(got, want.reshape(T, -1), 2e-4 if logits else 2e-5, "recurrence")
     assert float((state[1] - 7.0).abs().max()) == 0.0 and float(state[3].abs().max()) == 0.0, "other slots stay as they were"
 
 
