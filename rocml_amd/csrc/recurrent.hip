@@ -924,7 +924,7 @@ __device__ __forceinline__ void rc_store4(bf16_t* p, float a, float b, float c, 
 template <typename TO>
 __global__ void __launch_bounds__(RC_BLOCK)
 head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__ g, int ldg, int g_col0,
-                          const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps) {
+                          const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps, int silu) {
     int lane = threadIdx.x & (WAVE - 1);
     long long row = (long long)blockIdx.x * (RC_BLOCK / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -933,8 +933,9 @@ head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__
     int nv = dv / 4;
     const sc_f4* src = (const sc_f4*)(o + (size_t)row * dv);
     const sc_f4* gr = (const sc_f4*)(g + (size_t)t * ldg + g_col0 + (size_t)h * dv);
-    const sc_f4* wr = (const sc_f4*)(gain + (size_t)h * dv);
+    const sc_f4* wr = gain ? (const sc_f4*)(gain + (size_t)h * dv) : nullptr;
     const sc_f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const sc_f4 one4 = {1.f, 1.f, 1.f, 1.f};
     sc_f4 v[2], z[2], w[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -942,7 +943,7 @@ head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__
         bool ok = c < nv;
         v[k] = ok ? src[c] : zero4;
         z[k] = ok ? gr[c] : zero4;
-        w[k] = ok ? wr[c] : zero4;
+        w[k] = (ok && wr) ? wr[c] : one4;
     }
     float ss = 0.f;
 #pragma unroll
@@ -956,12 +957,54 @@ head_norm_gate_vec_kernel(const float* __restrict__ o, const float* __restrict__
         int c = lane + k * WAVE;
         if (c >= nv) continue;
         TO* dst = out + (size_t)row * dv + 4 * (size_t)c;
-        float r0 = v[k].x * inv * w[k].x * (1.0f / (1.0f + expf(-z[k].x)));
-        float r1 = v[k].y * inv * w[k].y * (1.0f / (1.0f + expf(-z[k].y)));
-        float r2 = v[k].z * inv * w[k].z * (1.0f / (1.0f + expf(-z[k].z)));
-        float r3 = v[k].w * inv * w[k].w * (1.0f / (1.0f + expf(-z[k].w)));
+        // (the gate: sigmoid(z), or z sigmoid(z))
+        float g0 = 1.0f / (1.0f + expf(-z[k].x)), g1 = 1.0f / (1.0f + expf(-z[k].y));
+        float g2 = 1.0f / (1.0f + expf(-z[k].z)), g3 = 1.0f / (1.0f + expf(-z[k].w));
+        if (silu) { g0 *= z[k].x; g1 *= z[k].y; g2 *= z[k].z; g3 *= z[k].w; }
+        float r0 = v[k].x * inv * w[k].x * g0;
+        float r1 = v[k].y * inv * w[k].y * g1;
+        float r2 = v[k].z * inv * w[k].z * g2;
+        float r3 = v[k].w * inv * w[k].w * g3;
         rc_store4(dst, r0, r1, r2, r3);
     }
+}
+
+// Heads of at most 128 values (multiples of 4): G lanes a head, a 16-byte piece a lane, 64 / G heads a wave, the sum of
+// squares across the G lanes; a wave per head would leave most of its lanes idle there.
+template <typename TO, int G>
+__global__ void __launch_bounds__(RC_BLOCK)
+head_norm_gate_pack_kernel(const float* __restrict__ o, const float* __restrict__ g, int ldg, int g_col0,
+                           const float* __restrict__ gain, TO* __restrict__ out, long long n_rows, int n_heads, int dv, float eps, int silu) {
+    long long row = ((long long)blockIdx.x * RC_BLOCK + threadIdx.x) / G;
+    int c = threadIdx.x % G;
+    bool ok = row < n_rows && 4 * c < dv;
+    long long t = ok ? row / n_heads : 0;
+    int h = ok ? (int)(row - t * n_heads) : 0;
+    const sc_f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const sc_f4 one4 = {1.f, 1.f, 1.f, 1.f};
+    sc_f4 v = ok ? *(const sc_f4*)(o + (size_t)row * dv + 4 * c) : zero4;
+    sc_f4 z = ok ? *(const sc_f4*)(g + (size_t)t * ldg + g_col0 + (size_t)h * dv + 4 * c) : zero4;
+    sc_f4 w = (ok && gain) ? *(const sc_f4*)(gain + (size_t)h * dv + 4 * c) : one4;
+    float ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+    if (!ok) return;
+    float g0 = 1.0f / (1.0f + expf(-z.x)), g1 = 1.0f / (1.0f + expf(-z.y));
+    float g2 = 1.0f / (1.0f + expf(-z.z)), g3 = 1.0f / (1.0f + expf(-z.w));
+    if (silu) { g0 *= z.x; g1 *= z.y; g2 *= z.z; g3 *= z.w; }
+    rc_store4(out + (size_t)row * dv + 4 * c, v.x * inv * w.x * g0, v.y * inv * w.y * g1, v.z * inv * w.z * g2, v.w * inv * w.w * g3);
+}
+
+template <typename TO>
+static void launch_head_norm_gate_pack(const float* o, const float* g, int ldg, int g_col0, const float* gain, TO* out, long long rows,
+                                       int n_heads, int dv, float eps, int silu, hipStream_t stream) {
+    int lanes = dv / 4 <= 4 ? 4 : dv / 4 <= 8 ? 8 : dv / 4 <= 16 ? 16 : 32;
+    int grid = ceil_div(rows * lanes, RC_BLOCK);
+    if (lanes == 4) head_norm_gate_pack_kernel<TO, 4><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, out, rows, n_heads, dv, eps, silu);
+    else if (lanes == 8) head_norm_gate_pack_kernel<TO, 8><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, out, rows, n_heads, dv, eps, silu);
+    else if (lanes == 16) head_norm_gate_pack_kernel<TO, 16><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, out, rows, n_heads, dv, eps, silu);
+    else head_norm_gate_pack_kernel<TO, 32><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, out, rows, n_heads, dv, eps, silu);
 }
 
 // gate_act: 0 the gate is sigmoid(g), 1 it is silu(g) = g sigmoid(g).  gain may be null (ones).
@@ -973,12 +1016,16 @@ ROCML_EXPORT int rocml_head_norm_gate(const float* o, const float* g, int ldg, i
     long long rows = (long long)n_tokens * n_heads;
     if (rows == 0) return 0;
     int grid = ceil_div(rows, RC_BLOCK / WAVE);
-    bool vec = gate_act == 0 && gain && dv % 4 == 0 && dv <= 8 * WAVE && ldg % 4 == 0 && g_col0 % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0 &&
+    bool vec = dv % 4 == 0 && dv <= 8 * WAVE && ldg % 4 == 0 && g_col0 % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0 &&
                (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0;
-    if (vec && out_dtype == ROCML_F32)
-        head_norm_gate_vec_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps);
+    if (vec && dv <= 128 && out_dtype == ROCML_F32)
+        launch_head_norm_gate_pack<float>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps, gate_act, stream);
+    else if (vec && dv <= 128 && out_dtype == ROCML_BF16)
+        launch_head_norm_gate_pack<bf16_t>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps, gate_act, stream);
+    else if (vec && out_dtype == ROCML_F32)
+        head_norm_gate_vec_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps, gate_act);
     else if (vec && out_dtype == ROCML_BF16)
-        head_norm_gate_vec_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps);
+        head_norm_gate_vec_kernel<bf16_t><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (bf16_t*)out, rows, n_heads, dv, eps, gate_act);
     else if (out_dtype == ROCML_F32)
         head_norm_gate_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(o, g, ldg, g_col0, gain, (float*)out, rows, n_heads, dv, eps, gate_act);
     else if (out_dtype == ROCML_BF16)
@@ -1107,18 +1154,20 @@ ROCML_EXPORT int rocml_gated_part_norm(const float* y, const float* z, int ldz, 
 // token's key and value: S <- diag(w_t) S + k_t v_t^T.  Two ways to read it:
 //   after the update (a retention):        o_t = S_t^T q_t, with w_t one constant per head;
 //   before it, with a bonus on the token:  o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t, with w_t per token and channel.
-// The columns of S (one per value) do not depend on each other: a block takes (sequence, head, 16 values), the 16
-// lanes of a row of lanes hold one column, lane l the R entries l R .. l R + R - 1, and add their parts of the dot
-// product with q across the row.  The tokens' rows (q, k, the decays and the block's 16 values) come in chunks of 16
-// tokens through LDS: every thread owns up to DS_SLOTS columns of a chunk's rows, requests the next chunk's numbers
-// into registers before it works on this one, and writes them to LDS when this one is done, so the walk over the
-// tokens waits for memory once.  Inside a chunk four tokens are worked on at a time (their cross-lane sums side by
-// side).  w_logit: the decays come as logits x and are exp(-exp(x + offset)), formed on the way into LDS.  The state
-// is stored column by column, [slot, head, dv, dk].  Everything is 32-bit.
-constexpr int DS_COLS = 16;      // values (columns of the state) per block
+// The columns of S (one per value) do not depend on each other: a block takes (sequence, head, 16 CPL values).  The
+// 16 lanes of a row of lanes hold CPL neighbouring columns, lane l the R entries l R .. l R + R - 1 of each: what a
+// lane reads of q, k and the decays serves CPL columns, which is what keeps the walk off the LDS's bandwidth.  The
+// tokens' rows (q, k, the decays and the block's values) come in chunks of 16 tokens through LDS: every thread owns
+// up to SLOTS columns of a chunk's rows, requests the next chunk's numbers into registers before it works on this
+// one, and writes them to LDS when this one is done, so the walk over the tokens waits for memory once.  Inside a
+// chunk four tokens are worked on at a time: their 4 CPL partial sums per lane are added across the row of lanes so
+// that every lane ends with one whole sum (halving exchanges), which it writes.  w_offset: the decays come as logits
+// x and are exp(-exp(x + offset)), formed on the way into LDS.  The state is stored column by column,
+// [slot, head, dv, dk].  Everything is 32-bit.
 constexpr int DS_LANES = 16;     // lanes that share a column
-constexpr int DS_THREADS = DS_COLS * DS_LANES;
-constexpr int DS_CHUNK = 16;     // tokens of a chunk
+constexpr int DS_GROUPS = 16;    // rows of lanes in a block
+constexpr int DS_THREADS = DS_GROUPS * DS_LANES;
+constexpr int DS_CHUNK = 16;     // tokens of a chunk (8: 4 to 7 % slower on 8 x 2,048 tokens, 32: 9 to 25 %)
 constexpr int DS_TOKENS = 4;     // tokens whose sums cross the lanes together
 
 struct DecayScanArgs {
@@ -1133,66 +1182,147 @@ struct DecayScanArgs {
     float* out; int n_heads; int dk; int dv;
 };
 
-__device__ __forceinline__ float ds_row_sum(float v) {
-    v += __shfl_xor(v, 1, 64);
-    v += __shfl_xor(v, 2, 64);
-    v += __shfl_xor(v, 4, 64);
-    v += __shfl_xor(v, 8, 64);
-    return v;
-}
-
-// R: entries of a column per lane (dk <= 16 R).  PER_TOKEN: a decay per token and channel (else one per head).
-template <int R, bool BONUS, bool PER_TOKEN>
+// R: entries of a column per lane (dk <= 16 R).  CPL: columns per lane.  BONUS: a decay per token and channel and a
+// bonus, the state read before its update; else one decay per head, the state read after it.
+// A token's row in LDS has a fixed layout, whatever dk: q, k (and the decays) padded to 16 R numbers each, the block's
+// 16 CPL values, and without BONUS the token's decay (the head's, or one for the rows beyond the sequence's last
+// token, which then leave the state as it is: with BONUS their decays are one and their keys zero).  A lane reads its
+// R numbers of each part as whole vectors at fixed offsets, without a bound to check.
+template <int R, int CPL, bool BONUS>
 __global__ void __launch_bounds__(DS_THREADS)
 decay_scan_kernel(DecayScanArgs a) {
-    constexpr int ARRAYS = PER_TOKEN ? 3 : 2;                       // q, k (and the decays), each dk wide, then 16 values
-    constexpr int MAX_ROW = ARRAYS * 16 * R + DS_COLS;
-    constexpr int DS_SLOTS = (MAX_ROW + DS_THREADS - 1) / DS_THREADS;
-    extern __shared__ float ds_rows[];                               // [DS_CHUNK][row]
+    constexpr int ARRAYS = BONUS ? 3 : 2;
+    constexpr int DKP = DS_LANES * R;
+    constexpr int TILE = DS_GROUPS * CPL;                            // columns of a block
+    constexpr int ROW = ARRAYS * DKP + TILE + (BONUS ? 0 : 4);
+    constexpr int SLOTS = (ROW + DS_THREADS - 1) / DS_THREADS;
+    constexpr int NV = DS_TOKENS * CPL;                              // sums of a lane per group of tokens
+    __shared__ __attribute__((aligned(16))) float ds_rows[DS_CHUNK * ROW];
     int b = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
     int tid = threadIdx.x;
     int l = tid % DS_LANES, c = tid / DS_LANES;
     int dk = a.dk;
-    int row = ARRAYS * dk + DS_COLS;
-    int col = tile * DS_COLS + c;
-    bool col_ok = col < a.dv;
+    int col0 = tile * TILE + c * CPL;
     int first = a.cu_seqlens[b], n = a.cu_seqlens[b + 1] - first;
+    float hd = BONUS ? 0.f : a.head_decay[h];
     // the columns of a chunk's rows that this thread brings in: where they come from, per slot
-    const float* src[DS_SLOTS];
-    int src_ld[DS_SLOTS];
-    float offset[DS_SLOTS];
-    bool is_logit[DS_SLOTS];
+    const float* src[SLOTS];
+    int src_ld[SLOTS];
+    float offset[SLOTS], beyond[SLOTS], fixed[SLOTS];
+    bool is_logit[SLOTS];
 #pragma unroll
-    for (int m = 0; m < DS_SLOTS; ++m) {
+    for (int m = 0; m < SLOTS; ++m) {
         int x = tid + m * DS_THREADS;
         src[m] = nullptr;
         src_ld[m] = 0;
         offset[m] = 0.f;
+        beyond[m] = 0.f;           // what rows beyond the sequence's last token hold
+        fixed[m] = 0.f;            // what a column without a source holds
         is_logit[m] = false;
-        if (x < dk) { src[m] = a.q + a.q_col0 + (size_t)h * dk + x; src_ld[m] = a.ldq; }
-        else if (x < 2 * dk) { src[m] = a.k + a.k_col0 + (size_t)h * dk + (x - dk); src_ld[m] = a.ldk; }
-        else if (PER_TOKEN && x < 3 * dk) {
-            src[m] = a.w + a.w_col0 + (size_t)h * dk + (x - 2 * dk);
-            src_ld[m] = a.ldw;
-            if (a.w_offset) { is_logit[m] = true; offset[m] = a.w_offset[(size_t)h * dk + (x - 2 * dk)]; }
-        } else if (x < row) {
-            int vc = tile * DS_COLS + (x - ARRAYS * dk);
+        int part = x / DKP, ch = x - part * DKP;
+        if (part < ARRAYS) {
+            if (ch < dk) {
+                size_t e = (size_t)h * dk + ch;
+                if (part == 0) { src[m] = a.q + a.q_col0 + e; src_ld[m] = a.ldq; }
+                else if (part == 1) { src[m] = a.k + a.k_col0 + e; src_ld[m] = a.ldk; }
+                else {
+                    src[m] = a.w + a.w_col0 + e;
+                    src_ld[m] = a.ldw;
+                    beyond[m] = 1.f;
+                    if (a.w_offset) { is_logit[m] = true; offset[m] = a.w_offset[e]; }
+                }
+            }
+        } else if (x < ARRAYS * DKP + TILE) {
+            int vc = tile * TILE + (x - ARRAYS * DKP);
             if (vc < a.dv) { src[m] = a.v + a.v_col0 + (size_t)h * a.dv + vc; src_ld[m] = a.ldv; }
+        } else {
+            fixed[m] = hd;
+            beyond[m] = 1.f;
         }
     }
-    float* st = a.state + (((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv + (col_ok ? col : 0)) * dk;
-    float s[R], u[R];
+    float* st = a.state + ((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv * dk;
+    float s[CPL][R], u[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int i = l * R + r;
-        s[r] = (col_ok && i < dk) ? st[i] : 0.f;
         u[r] = (BONUS && i < dk) ? a.bonus[(size_t)h * dk + i] : 0.f;
+#pragma unroll
+        for (int p = 0; p < CPL; ++p) s[p][r] = (col0 + p < a.dv && i < dk) ? st[(size_t)(col0 + p) * dk + i] : 0.f;
     }
-    float hd = PER_TOKEN ? 0.f : a.head_decay[h];
-    float next[DS_SLOTS][DS_CHUNK];
+    // what a token does to the lane's columns: qq, kk, ww the lane's R numbers of the token's rows, vv its columns' values
+    auto token = [&](const float (&qq)[R], const float (&kk)[R], const float (&ww)[R], const float (&vv)[CPL], float dec, float* sums) {
+        if constexpr (BONUS) {
+            // (S + diag(u) k v^T)^T q = S^T q + v (u . k q): the second part is the same for every column
+            float ukq = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) ukq = fmaf(u[r] * kk[r], qq[r], ukq);
+#pragma unroll
+            for (int p = 0; p < CPL; ++p) {
+                float sum = ukq * vv[p];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    sum = fmaf(s[p][r], qq[r], sum);
+                    s[p][r] = fmaf(ww[r], s[p][r], kk[r] * vv[p]);
+                }
+                sums[p] = sum;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < CPL; ++p) {
+                float sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    s[p][r] = fmaf(dec, s[p][r], kk[r] * vv[p]);
+                    sum = fmaf(s[p][r], qq[r], sum);
+                }
+                sums[p] = sum;
+            }
+        }
+    };
+    auto keep_state = [&]() {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int i = l * R + r;
+#pragma unroll
+            for (int p = 0; p < CPL; ++p)
+                if (col0 + p < a.dv && i < dk) st[(size_t)(col0 + p) * dk + i] = s[p][r];
+        }
+    };
+    if (n == 1) {
+        // One token (a decode step): its numbers come straight from memory, beside the state's; the same arithmetic.
+        float qq[R], kk[R], ww[R], vv[CPL], sums[CPL];
+        size_t t = (size_t)first;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int i = l * R + r;
+            bool in = i < dk;
+            size_t e = (size_t)h * dk + i;
+            qq[r] = in ? a.q[t * a.ldq + a.q_col0 + e] : 0.f;
+            kk[r] = in ? a.k[t * a.ldk + a.k_col0 + e] : 0.f;
+            ww[r] = 0.f;
+            if constexpr (BONUS) {
+                if (in) {
+                    float x = a.w[t * a.ldw + a.w_col0 + e];
+                    ww[r] = a.w_offset ? expf(-expf(x + a.w_offset[e])) : x;
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < CPL; ++p) vv[p] = col0 + p < a.dv ? a.v[t * a.ldv + a.v_col0 + (size_t)h * a.dv + col0 + p] : 0.f;
+        token(qq, kk, ww, vv, hd, sums);
+#pragma unroll
+        for (int p = 0; p < CPL; ++p) sums[p] = row16_sum(sums[p]);
+        float out_val = sums[0];
+#pragma unroll
+        for (int p = 1; p < CPL; ++p) out_val = l == p ? sums[p] : out_val;
+        if (l < CPL && col0 + l < a.dv) a.out[t * a.n_heads * a.dv + (size_t)h * a.dv + col0 + l] = out_val;
+        keep_state();
+        return;
+    }
+    float next[SLOTS][DS_CHUNK];
     auto request = [&](int t0) {
 #pragma unroll
-        for (int m = 0; m < DS_SLOTS; ++m)
+        for (int m = 0; m < SLOTS; ++m)
 #pragma unroll
             for (int j = 0; j < DS_CHUNK; ++j)
                 next[m][j] = (src[m] && t0 + j < n) ? src[m][(size_t)(first + t0 + j) * src_ld[m]] : 0.f;
@@ -1200,74 +1330,90 @@ decay_scan_kernel(DecayScanArgs a) {
     request(0);
     for (int t0 = 0; t0 < n; t0 += DS_CHUNK) {
 #pragma unroll
-        for (int m = 0; m < DS_SLOTS; ++m) {
+        for (int m = 0; m < SLOTS; ++m) {
             int x = tid + m * DS_THREADS;
-            if (x < row) {
+            if (x < ROW) {
 #pragma unroll
                 for (int j = 0; j < DS_CHUNK; ++j) {
                     float val = next[m][j];
-                    if (PER_TOKEN && is_logit[m]) val = expf(-expf(val + offset[m]));
-                    ds_rows[j * row + x] = val;
+                    if (BONUS && is_logit[m]) val = expf(-expf(val + offset[m]));
+                    if (!src[m]) val = fixed[m];
+                    if (t0 + j >= n) val = beyond[m];
+                    ds_rows[j * ROW + x] = val;
                 }
             }
         }
         __syncthreads();
         if (t0 + DS_CHUNK < n) request(t0 + DS_CHUNK);
         int here = min(DS_CHUNK, n - t0);
+        const float* mine = ds_rows + l * R;
         for (int j0 = 0; j0 < here; j0 += DS_TOKENS) {
-            float acc[DS_TOKENS];
+            float acc[NV];
 #pragma unroll
             for (int jj = 0; jj < DS_TOKENS; ++jj) {
-                const float* tok = ds_rows + (j0 + jj) * row;
-                float sum = 0.f;
-                if (j0 + jj < here) {
-                    float vv = tok[ARRAYS * dk + c];
+                const float* tok = mine + (j0 + jj) * ROW;
+                float qq[R], kk[R], ww[R], vv[CPL];
+                if constexpr (R % 4 == 0) {
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        int i = l * R + r;
-                        bool in = i < dk;
-                        float qq = in ? tok[i] : 0.f;
-                        float kv = (in ? tok[dk + i] : 0.f) * vv;
-                        float ww = PER_TOKEN ? (in ? tok[2 * dk + i] : 0.f) : hd;
+                    for (int r4 = 0; r4 < R / 4; ++r4) {
+                        float4 q4 = *(const float4*)(tok + 4 * r4);
+                        float4 k4 = *(const float4*)(tok + DKP + 4 * r4);
+                        qq[4 * r4] = q4.x; qq[4 * r4 + 1] = q4.y; qq[4 * r4 + 2] = q4.z; qq[4 * r4 + 3] = q4.w;
+                        kk[4 * r4] = k4.x; kk[4 * r4 + 1] = k4.y; kk[4 * r4 + 2] = k4.z; kk[4 * r4 + 3] = k4.w;
                         if constexpr (BONUS) {
-                            sum = fmaf(fmaf(u[r], kv, s[r]), qq, sum);
-                            s[r] = fmaf(ww, s[r], kv);
-                        } else {
-                            s[r] = fmaf(ww, s[r], kv);
-                            sum = fmaf(s[r], qq, sum);
+                            float4 w4 = *(const float4*)(tok + 2 * DKP + 4 * r4);
+                            ww[4 * r4] = w4.x; ww[4 * r4 + 1] = w4.y; ww[4 * r4 + 2] = w4.z; ww[4 * r4 + 3] = w4.w;
                         }
                     }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        qq[r] = tok[r];
+                        kk[r] = tok[DKP + r];
+                        if constexpr (BONUS) ww[r] = tok[2 * DKP + r];
+                    }
                 }
-                acc[jj] = sum;
+                const float* vals = ds_rows + (j0 + jj) * ROW + ARRAYS * DKP;
+                if constexpr (CPL == 4) {
+                    float4 v4 = *(const float4*)(vals + c * CPL);
+                    vv[0] = v4.x; vv[1] = v4.y; vv[2] = v4.z; vv[3] = v4.w;
+                } else {
+#pragma unroll
+                    for (int p = 0; p < CPL; ++p) vv[p] = vals[c * CPL + p];
+                }
+                float dec = 0.f;
+                if constexpr (!BONUS) dec = vals[TILE];
+                token(qq, kk, ww, vv, dec, acc + jj * CPL);
             }
 #pragma unroll
-            for (int jj = 0; jj < DS_TOKENS; ++jj) acc[jj] = ds_row_sum(acc[jj]);
-            if (l < DS_TOKENS && col_ok) {
-                float mine = acc[0];
+            for (int i = 0; i < NV; ++i) acc[i] = row16_sum(acc[i]);
+            float out_val = acc[0];
 #pragma unroll
-                for (int jj = 1; jj < DS_TOKENS; ++jj) mine = l == jj ? acc[jj] : mine;
-                if (j0 + l < here) a.out[(size_t)(first + t0 + j0 + l) * a.n_heads * a.dv + (size_t)h * a.dv + col] = mine;
-            }
+            for (int i = 1; i < NV; ++i) out_val = l == i ? acc[i] : out_val;
+            int jj = l / CPL, p = l - jj * CPL;
+            if (l < NV && j0 + jj < here && col0 + p < a.dv)
+                a.out[(size_t)(first + t0 + j0 + jj) * a.n_heads * a.dv + (size_t)h * a.dv + col0 + p] = out_val;
         }
         __syncthreads();                         // the rows are rewritten by the next chunk
     }
-    if (col_ok) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int i = l * R + r;
-            if (i < dk) st[i] = s[r];
-        }
-    }
+    keep_state();
+}
+
+template <int R, int CPL>
+static void launch_decay_scan_cols(const DecayScanArgs& a, int n_seqs, hipStream_t stream) {
+    dim3 grid(n_seqs, a.n_heads, ceil_div(a.dv, DS_GROUPS * CPL));
+    if (a.bonus) decay_scan_kernel<R, CPL, true><<<grid, DS_THREADS, 0, stream>>>(a);
+    else decay_scan_kernel<R, CPL, false><<<grid, DS_THREADS, 0, stream>>>(a);
 }
 
 template <int R>
 static void launch_decay_scan(const DecayScanArgs& a, int n_seqs, hipStream_t stream) {
-    dim3 grid(n_seqs, a.n_heads, ceil_div(a.dv, DS_COLS));
-    size_t lds = (size_t)DS_CHUNK * ((a.w ? 3 : 2) * a.dk + DS_COLS) * sizeof(float);
-    if (a.w && a.bonus) decay_scan_kernel<R, true, true><<<grid, DS_THREADS, lds, stream>>>(a);
-    else if (a.w) decay_scan_kernel<R, false, true><<<grid, DS_THREADS, lds, stream>>>(a);
-    else if (a.bonus) decay_scan_kernel<R, true, false><<<grid, DS_THREADS, lds, stream>>>(a);
-    else decay_scan_kernel<R, false, false><<<grid, DS_THREADS, lds, stream>>>(a);
+        // Two columns per lane (a lane's reads of q, k and the decays then serve both) where blocks of 16 columns would be
+    // more than two a CU: measured on 8 x 2,048 tokens of 32 heads of 64 x 64 at 0.76 ms against 1.06 with one column
+    // and 0.76 with four; a single sequence, whose blocks are fewer than the CUs, is faster with one (0.47 against 0.52).
+    long long blocks = (long long)n_seqs * a.n_heads * ceil_div(a.dv, DS_GROUPS);
+    if (R <= 8 && a.dv > DS_GROUPS && blocks > 2ll * cu_count()) launch_decay_scan_cols<R, R <= 8 ? 2 : 1>(a, n_seqs, stream);
+    else launch_decay_scan_cols<R, 1>(a, n_seqs, stream);
 }
 
 ROCML_EXPORT int rocml_decay_scan(const float* q, int ldq, int q_col0, const float* k, int ldk, int k_col0, const float* v,
@@ -1279,7 +1425,8 @@ ROCML_EXPORT int rocml_decay_scan(const float* q, int ldq, int q_col0, const flo
                   n_tokens, n_seqs, n_heads);
     ROCML_REQUIRE(dk <= 16 * DS_LANES, "decay_scan: a key size of %d exceeds %d", dk, 16 * DS_LANES);
     ROCML_REQUIRE(q && k && v && state && cu_seqlens && seq_slots && out, "decay_scan: missing arguments");
-    ROCML_REQUIRE((w != nullptr) != (head_decay != nullptr), "decay_scan: a decay per token and channel or one per head, one of the two");
+    ROCML_REQUIRE((w != nullptr) != (head_decay != nullptr) && (w != nullptr) == (bonus != nullptr),
+                  "decay_scan: a decay per token and channel with a bonus, or one decay per head without");
     ROCML_REQUIRE(!w_offset || w, "decay_scan: an offset goes with decays given as logits");
     ROCML_REQUIRE(q_col0 >= 0 && k_col0 >= 0 && v_col0 >= 0 && ldq >= q_col0 + n_heads * dk && ldk >= k_col0 + n_heads * dk &&
                       ldv >= v_col0 + n_heads * dv && (!w || (w_col0 >= 0 && ldw >= w_col0 + n_heads * dk)),
@@ -1300,10 +1447,11 @@ ROCML_EXPORT int rocml_decay_scan(const float* q, int ldq, int q_col0, const flo
 // ---- rotation of heads inside a 32-bit matrix --------------------------------------------
 // Columns col0 .. col0 + n_heads * d - 1 of buf [T, ld]: of every head the first `rot` numbers turn, number i with
 // number i + rot/2 by the angle whose cosine and sine stand in column i of the tables [T, rot/2]; then every number
-// of the heads is multiplied by `scale`.  In place; a thread owns a pair (or one number beyond the rotated part).
+// of the heads is multiplied by `scale` (heads from `heads_first` on by `scale_rest`: queries and keys that lie side by
+// side go through one launch).  In place; a thread owns a pair (or one number beyond the rotated part).
 __global__ void __launch_bounds__(RC_BLOCK)
 rotate_rows_kernel(float* __restrict__ buf, int ld, int col0, int n_heads, int d, int rot, const float* __restrict__ cos_t,
-                   const float* __restrict__ sin_t, float scale, long long total) {
+                   const float* __restrict__ sin_t, float scale, int heads_first, float scale_rest, long long total) {
     long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
     if (idx >= total) return;
     int half = rot / 2, per_head = d - half;
@@ -1312,6 +1460,7 @@ rotate_rows_kernel(float* __restrict__ buf, int ld, int col0, int n_heads, int d
     long long t = th / n_heads;
     int h = (int)(th - t * n_heads);
     float* row = buf + (size_t)t * ld + col0 + (size_t)h * d;
+    if (h >= heads_first) scale = scale_rest;
     if (e < half) {
         float c = cos_t[(size_t)t * half + e], s = sin_t[(size_t)t * half + e];
         float x = row[e], y = row[e + half];
@@ -1323,13 +1472,14 @@ rotate_rows_kernel(float* __restrict__ buf, int ld, int col0, int n_heads, int d
 }
 
 ROCML_EXPORT int rocml_rotate_rows(float* buf, int ld, int col0, int n_tokens, int n_heads, int d, int rot, const float* cos_t,
-                                   const float* sin_t, float scale, hipStream_t stream) {
+                                   const float* sin_t, float scale, int heads_first, float scale_rest, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && d > 0 && rot >= 0 && rot % 2 == 0 && rot <= d, "rotate_rows: bad sizes heads=%d d=%d rot=%d",
                   n_heads, d, rot);
     ROCML_REQUIRE(buf && col0 >= 0 && ld >= col0 + n_heads * d && (rot == 0 || (cos_t && sin_t)), "rotate_rows: bad arguments");
     long long total = (long long)n_tokens * n_heads * (d - rot / 2);
     if (total == 0) return 0;
-    rotate_rows_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(buf, ld, col0, n_heads, d, rot, cos_t, sin_t, scale, total);
+    rotate_rows_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(buf, ld, col0, n_heads, d, rot, cos_t, sin_t, scale,
+                                                                           heads_first, scale_rest, total);
     ROCML_CHECK_LAUNCH("rotate_rows");
     return 0;
 }

@@ -61,7 +61,7 @@ _SIGNATURES = {
         "rocml_mlstm_tile": [],
         "rocml_head_norm_gate": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
         "rocml_decay_scan": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _P],
-        "rocml_rotate_rows": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P],
+        "rocml_rotate_rows": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _I, _F, _P],
         "rocml_shift_mix": [_P, _I, _I, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P],
         "rocml_tanh": [_P, _P, _I, _LL, _P],
         "rocml_double_exp_decay": [_P, _P, _I, _I, _P],
@@ -1283,10 +1283,10 @@ def decay_scan(q: torch.Tensor, q_col0: int, k: torch.Tensor, k_col0: int, v: to
 
 
 def rotate_rows(buf: torch.Tensor, col0: int, n_heads: int, head_dim: int, rot_dim: int, cos: Optional[torch.Tensor],
-                sin: Optional[torch.Tensor], scale: float = 1.0) -> None:
+                sin: Optional[torch.Tensor], scale: float = 1.0, heads_first: Optional[int] = None, scale_rest: float = 1.0) -> None:
     """In place on columns ``col0 .. col0 + n_heads * head_dim - 1`` of the 32-bit ``buf [T, ld]``: of every head the
     first ``rot_dim`` numbers turn (number ``i`` with ``i + rot_dim / 2``, angles from the tables ``[T, rot_dim / 2]``),
-    then the heads are multiplied by ``scale``."""
+    then the heads are multiplied by ``scale`` (with ``heads_first``: the heads from that one on by ``scale_rest``)."""
     _dev(buf, cos, sin)
     _want(buf, torch.float32, "the matrix to rotate")
     n_tokens = buf.shape[0]
@@ -1294,7 +1294,9 @@ def rotate_rows(buf: torch.Tensor, col0: int, n_heads: int, head_dim: int, rot_d
         if cos is None or sin is None or cos.shape != (n_tokens, rot_dim // 2) or sin.shape != cos.shape:
             raise KernelError(f"rotation tables must be {(n_tokens, rot_dim // 2)}")
     _check("recurrent", library("recurrent").rocml_rotate_rows(_ptr(buf), buf.shape[1], col0, n_tokens, n_heads, head_dim, rot_dim,
-                                                             _ptr(cos), _ptr(sin), float(scale), _stream()))
+                                                             _ptr(cos), _ptr(sin), float(scale),
+                                                             n_heads if heads_first is None else int(heads_first), float(scale_rest),
+                                                             _stream()))
 
 
 def shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor,

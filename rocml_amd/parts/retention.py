@@ -88,10 +88,9 @@ class Retention(Mixer):
         if self.position is not None:
             cos, sin = self.position.tables(step)
             rot = self.position.rot_dim
-        # q and k are neighbours in the projection: both rotated in one launch, then k scaled by itself
-        if rot:
-            ops.rotate_rows(proj, 0, 2 * s.n_heads, s.head_dim, rot, cos, sin, 1.0)
-        ops.rotate_rows(proj, self.k_col, s.n_heads, s.head_dim, 0, None, None, float(s.head_dim) ** -0.5)
+        # q and k are neighbours in the projection: both rotated in one launch, in which the k heads are scaled too
+        ops.rotate_rows(proj, 0, 2 * s.n_heads, s.head_dim, rot, cos, sin, 1.0, heads_first=s.n_heads,
+                        scale_rest=float(s.head_dim) ** -0.5)
         o = ws.get("retention.o", (n, self.v_dim), torch.float32)
         ops.decay_scan(proj, 0, proj, self.k_col, proj, self.v_col, cache.state, step.cu_seqlens, step.seq_slots, o,
                        s.n_heads, s.head_dim, s.v_head_dim, head_decay=self.decay)

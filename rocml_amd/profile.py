@@ -165,7 +165,7 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
                        + 2 * slots.numel() * n_heads * head_dim * v_head_dim * 4,
                        (6 if kw.get("bonus") is not None else 4) * out.shape[0] * n_heads * head_dim * v_head_dim,
                        PEAK_FLOPS[torch.float32])),
-    "rotate_rows": ("rotation inside the projection", lambda buf, col0, n_heads, head_dim, rot_dim, cos, sin, scale=1.0: (
+    "rotate_rows": ("rotation inside the projection", lambda buf, col0, n_heads, head_dim, rot_dim, cos, sin, scale=1.0, **kw: (
         2 * buf.shape[0] * n_heads * head_dim * 4 + _nbytes(cos, sin), 3 * buf.shape[0] * n_heads * head_dim)),
     "shift_mix": ("mixes with the previous token", lambda h, mu, state, token_seq, cu, slots, out: (_nbytes(h, mu, out), 2 * out.numel())),
     "tanh": ("tanh between the decay's matrices", lambda x, out: (_nbytes(x, out), 10 * x.numel())),
