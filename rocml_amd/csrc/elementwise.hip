@@ -1278,12 +1278,14 @@ ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float 
 // ---- norm of a sublayer's output, added to the stream ------------------------------------------
 // x[t, :] += f(y[t, :]) in 32-bit, f a layer norm, (y - mean) / sqrt(var + eps) * gain + bias with var the mean
 // of the squared deviations from the mean (LAYER), or y / sqrt(mean(y^2) + eps) * gain; `copy` (may be null) gets
-// the new x in another type, for the products that read it next.  One block per row.
+// the new x in another type, for the products that read it next; with next_gain it gets the root-mean-square norm
+// of the new x instead, x / sqrt(mean(x^2) + next_eps) * next_gain: the norm that reads the stream next.  One block per row.
 template <typename TC, bool LAYER>
 __global__ void __launch_bounds__(EW_BLOCK)
 norm_add_kernel(float* __restrict__ x, float* __restrict__ y, const float* __restrict__ gain,
                 const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy,
-                const float* __restrict__ partials, int n_splits, long long split_stride, int replace) {
+                const float* __restrict__ partials, int n_splits, long long split_stride, int replace,
+                const float* __restrict__ next_gain, float next_eps) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     size_t row = (size_t)blockIdx.x * n;
     if (n_splits > 0) {         // y (or nothing) plus the K pieces in split order, written back: a thread reads back its own
@@ -1310,7 +1312,13 @@ norm_add_kernel(float* __restrict__ x, float* __restrict__ y, const float* __res
         if (LAYER && bias) v += bias[i];
         v += x[row + i];
         x[row + i] = v;
-        if (copy) Elem<TC>::store(copy + row + i, v);
+        if (copy && !next_gain) Elem<TC>::store(copy + row + i, v);
+    }
+    if (copy && next_gain) {        // (a thread reads back what it wrote itself)
+        float s2 = 0.f;
+        for (int i = threadIdx.x; i < n; i += EW_BLOCK) s2 = fmaf(x[row + i], x[row + i], s2);
+        float inv2 = 1.0f / sqrtf(block_sum(s2, scratch) / (float)n + next_eps);
+        for (int i = threadIdx.x; i < n; i += EW_BLOCK) Elem<TC>::store(copy + row + i, x[row + i] * inv2 * next_gain[i]);
     }
 }
 
@@ -1320,7 +1328,8 @@ template <typename TC, bool LAYER, int VEC>
 __global__ void __launch_bounds__(EW_BLOCK)
 norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
                     const float* __restrict__ bias, float eps, int n, TC* __restrict__ copy,
-                    const float* __restrict__ partials, int n_splits, long long split_stride, int replace) {
+                    const float* __restrict__ partials, int n_splits, long long split_stride, int replace,
+                    const float* __restrict__ next_gain, float next_eps) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     size_t row = (size_t)blockIdx.x * n;
     int nv = n / 4;
@@ -1373,19 +1382,39 @@ norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y, const fl
         v.z = xv[j].z + (yv[j].z * inv * gv[j].z + bv[j].z);
         v.w = xv[j].w + (yv[j].w * inv * gv[j].w + bv[j].w);
         ((float4*)(x + row))[i] = v;
-        if (copy) store4(copy + row + 4 * (size_t)i, v.x, v.y, v.z, v.w);
+        if (copy && !next_gain) store4(copy + row + 4 * (size_t)i, v.x, v.y, v.z, v.w);
+        xv[j] = v;
+    }
+    if (copy && next_gain) {        // the norm that reads the stream next, from the row in registers
+        float s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if (threadIdx.x + j * EW_BLOCK >= nv) continue;
+            s2 = fmaf(xv[j].x, xv[j].x, s2); s2 = fmaf(xv[j].y, xv[j].y, s2);
+            s2 = fmaf(xv[j].z, xv[j].z, s2); s2 = fmaf(xv[j].w, xv[j].w, s2);
+        }
+        float inv2 = 1.0f / sqrtf(block_sum(s2, scratch) / (float)n + next_eps);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            int i = threadIdx.x + j * EW_BLOCK;
+            if (i >= nv) continue;
+            float4 g2 = ((const float4*)next_gain)[i];
+            store4(copy + row + 4 * (size_t)i, xv[j].x * inv2 * g2.x, xv[j].y * inv2 * g2.y, xv[j].z * inv2 * g2.z, xv[j].w * inv2 * g2.w);
+        }
     }
 }
 
 template <typename TC, bool LAYER>
 static void launch_norm_add(float* x, float* y, const float* gain, const float* bias, float eps, int n_rows, int n,
-                            TC* copy, const float* partials, int n_splits, long long split_stride, int replace, hipStream_t stream) {
+                            TC* copy, const float* partials, int n_splits, long long split_stride, int replace,
+                            const float* next_gain, float next_eps, hipStream_t stream) {
     bool vec = n % 4 == 0 && n <= 4 * EW_BLOCK * RN_MAX_VEC && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
                (uintptr_t)gain % 16 == 0 && (!bias || (uintptr_t)bias % 16 == 0) && (!copy || (uintptr_t)copy % 8 == 0) &&
+               (!next_gain || (uintptr_t)next_gain % 16 == 0) &&
                (n_splits == 0 || ((uintptr_t)partials % 16 == 0 && split_stride % 4 == 0));
     int v = ceil_div(n / 4, EW_BLOCK);
-#define NAV(V_) norm_add_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace)
-    if (!vec) norm_add_kernel<TC, LAYER><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace);
+#define NAV(V_) norm_add_vec_kernel<TC, LAYER, V_><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace, next_gain, next_eps)
+    if (!vec) norm_add_kernel<TC, LAYER><<<n_rows, EW_BLOCK, 0, stream>>>(x, y, gain, bias, eps, n, copy, partials, n_splits, split_stride, replace, next_gain, next_eps);
     else if (v <= 1) NAV(1);
     else if (v <= 2) NAV(2);
     else if (v <= 4) NAV(4);
@@ -1509,7 +1538,9 @@ ROCML_EXPORT int rocml_norm_add_branches(float* x, const float* y0, const float*
 
 ROCML_EXPORT int rocml_norm_add(float* x, float* y, int n_rows, int n, const float* gain, const float* bias,
                                 float eps, int layer, void* copy, int copy_dtype, const float* partials, int n_splits,
-                                long long split_stride, int replace, hipStream_t stream) {
+                                long long split_stride, int replace, const float* next_gain, float next_eps, hipStream_t stream) {
+    // next_gain (may be null; needs copy): copy gets the new x normed, x / sqrt(mean(x^2) + next_eps) * next_gain
+    ROCML_REQUIRE(!next_gain || copy, "norm_add: the next norm's output needs a place");
     // layer = 1: layer norm (mean taken off, bias added if given); 0: root-mean-square norm (bias is not read)
     // partials (may be null): [n_splits][rows][n] K pieces of the product that made y, added to y in split order first;
     // with replace they are all of y (what y holds is not read; the plain kernel uses y as its buffer)
@@ -1520,11 +1551,11 @@ ROCML_EXPORT int rocml_norm_add(float* x, float* y, int n_rows, int n, const flo
     if (n_rows == 0) return 0;
     bool half = copy && copy_dtype == ROCML_BF16;
     if (layer) {
-        if (half) launch_norm_add<bf16_t, true>(x, y, gain, bias, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, stream);
-        else launch_norm_add<float, true>(x, y, gain, bias, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, stream);
+        if (half) launch_norm_add<bf16_t, true>(x, y, gain, bias, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, next_gain, next_eps, stream);
+        else launch_norm_add<float, true>(x, y, gain, bias, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, next_gain, next_eps, stream);
     } else {
-        if (half) launch_norm_add<bf16_t, false>(x, y, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, stream);
-        else launch_norm_add<float, false>(x, y, gain, nullptr, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, stream);
+        if (half) launch_norm_add<bf16_t, false>(x, y, gain, nullptr, eps, n_rows, n, (bf16_t*)copy, partials, n_splits, split_stride, replace, next_gain, next_eps, stream);
+        else launch_norm_add<float, false>(x, y, gain, nullptr, eps, n_rows, n, (float*)copy, partials, n_splits, split_stride, replace, next_gain, next_eps, stream);
     }
     ROCML_CHECK_LAUNCH("norm_add");
     return 0;

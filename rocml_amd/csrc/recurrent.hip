@@ -1242,12 +1242,32 @@ decay_scan_kernel(DecayScanArgs a) {
     }
     float* st = a.state + ((size_t)a.seq_slots[b] * a.n_heads + h) * a.dv * dk;
     float s[CPL][R], u[R];
+    // (a lane's R entries of a column lie side by side: 16-byte pieces where the sizes allow)
+    bool wide = R % 4 == 0 && dk % 4 == 0 && ((uintptr_t)a.state & 15) == 0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int i = l * R + r;
         u[r] = (BONUS && i < dk) ? a.bonus[(size_t)h * dk + i] : 0.f;
+    }
+    if (wide) {
+        if constexpr (R % 4 == 0) {
 #pragma unroll
-        for (int p = 0; p < CPL; ++p) s[p][r] = (col0 + p < a.dv && i < dk) ? st[(size_t)(col0 + p) * dk + i] : 0.f;
+            for (int p = 0; p < CPL; ++p)
+#pragma unroll
+                for (int r4 = 0; r4 < R / 4; ++r4) {
+                    int i = l * R + 4 * r4;
+                    float4 z = {0.f, 0.f, 0.f, 0.f};
+                    float4 v4 = (col0 + p < a.dv && i < dk) ? *(const float4*)(st + (size_t)(col0 + p) * dk + i) : z;
+                    s[p][4 * r4] = v4.x; s[p][4 * r4 + 1] = v4.y; s[p][4 * r4 + 2] = v4.z; s[p][4 * r4 + 3] = v4.w;
+                }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int i = l * R + r;
+#pragma unroll
+            for (int p = 0; p < CPL; ++p) s[p][r] = (col0 + p < a.dv && i < dk) ? st[(size_t)(col0 + p) * dk + i] : 0.f;
+        }
     }
     // what a token does to the lane's columns: qq, kk, ww the lane's R numbers of the token's rows, vv its columns' values
     auto token = [&](const float (&qq)[R], const float (&kk)[R], const float (&ww)[R], const float (&vv)[CPL], float dec, float* sums) {
@@ -1280,6 +1300,19 @@ decay_scan_kernel(DecayScanArgs a) {
         }
     };
     auto keep_state = [&]() {
+        if (wide) {
+            if constexpr (R % 4 == 0) {
+#pragma unroll
+                for (int p = 0; p < CPL; ++p)
+#pragma unroll
+                    for (int r4 = 0; r4 < R / 4; ++r4) {
+                        int i = l * R + 4 * r4;
+                        if (col0 + p < a.dv && i < dk)
+                            *(float4*)(st + (size_t)(col0 + p) * dk + i) = float4{s[p][4 * r4], s[p][4 * r4 + 1], s[p][4 * r4 + 2], s[p][4 * r4 + 3]};
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             int i = l * R + r;

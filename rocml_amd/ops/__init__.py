@@ -34,7 +34,7 @@ _SIGNATURES = {
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
                                       _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P, _I, _P],
         "rocml_qk_span_stats": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _P],
-        "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P, _I, _LL, _I, _P],
+        "rocml_norm_add": [_P, _P, _I, _I, _P, _P, _F, _I, _P, _I, _P, _I, _LL, _I, _P, _F, _P],
         "rocml_norm_add_branches": [_P, _P, _P, _P, _P, _F, _F, _I, _I, _P, _P, _F, _I, _P, _I, _P],
         "rocml_norm_add_branches_fits": [_I],
         "rocml_layernorm": [_P, _P, _I, _I, _P, _P, _F, _P, _I, _P],
@@ -375,12 +375,16 @@ def qk_span_stats(qkv: torch.Tensor, q_width: int, k_width: int, bias: Optional[
 
 def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
              layer: bool, copy: Optional[torch.Tensor] = None, partials: Optional[torch.Tensor] = None,
-             replace: bool = False) -> None:
+             replace: bool = False, next_gain: Optional[torch.Tensor] = None, next_eps: float = 0.0) -> None:
     """``x += f(y)`` row by row in 32-bit: ``f`` a layer norm ``(y - mean) / sqrt(var + eps) * gain + bias``
     (``layer``) or ``y / sqrt(mean(y^2) + eps) * gain``.  ``copy`` gets the new ``x`` in its own type.
     ``partials`` (``[splits, rows, n]`` 32-bit): the K pieces of the product that made ``y``, added to ``y`` in
-    split order first, or with ``replace`` all of ``y`` (what ``y`` holds is not read)."""
-    _dev(x, y, gain, bias, copy, partials)
+    split order first, or with ``replace`` all of ``y`` (what ``y`` holds is not read).  ``next_gain`` (with ``copy``):
+    ``copy`` gets the root-mean-square norm of the new ``x`` instead, ``x / sqrt(mean(x^2) + next_eps) * next_gain``: the
+    norm that reads the stream next."""
+    _dev(x, y, gain, bias, copy, partials, next_gain)
+    if next_gain is not None and (copy is None or next_gain.dtype != torch.float32 or next_gain.numel() != x.shape[1]):
+        raise KernelError("norm_add: the next norm needs a 32-bit gain of the row's size and a place for its output")
     n_splits = split_stride = 0
     if partials is not None:
         _want(partials, torch.float32, "partial sums")
@@ -396,7 +400,8 @@ def norm_add(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, bias: Optiona
         raise KernelError("norm_add: shapes do not fit")
     _check("elementwise", library("elementwise").rocml_norm_add(
         _ptr(x), _ptr(y), x.shape[0], x.shape[1], _ptr(gain), _ptr(bias), float(eps), 1 if layer else 0, _ptr(copy),
-        _code(copy) if copy is not None else 0, _ptr(partials), n_splits, split_stride, 1 if replace else 0, _stream()))
+        _code(copy) if copy is not None else 0, _ptr(partials), n_splits, split_stride, 1 if replace else 0, _ptr(next_gain),
+        float(next_eps), _stream()))
 
 
 def norm_add_branches_fits(n: int, n_branches: int) -> bool:

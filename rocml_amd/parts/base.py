@@ -138,6 +138,12 @@ class NormHint:
     width: int
 
 
+@dataclass(frozen=True)
+class FullNormHint(NormHint):
+    """The same norm, for a consumer that wants the norm's whole output (not an operand that still lacks its rows' scale):
+    a kernel that completes the stream may write ``x / sqrt(mean(x^2) + eps) * gain`` in the compute type beside it."""
+
+
 class Norm(Part):
     fuses_pending = False     # True: forward() takes ``pending`` partial sums and adds them to x itself
 

@@ -19,7 +19,7 @@ import torch
 
 from ..config.spec import BlockSpec
 from ..errors import ConfigError
-from .base import BuildContext, ParamSpec, Part
+from .base import BuildContext, FullNormHint, ParamSpec, Part
 from .registry import build_feed_forward, build_mixer, build_norm, register_block
 from .residual import stream
 
@@ -320,10 +320,13 @@ class SandwichNormBlock(Part):
     """``x += out_norm1(mixer(norm1(x)))``, ``x += out_norm2(ffn(norm2(x)))``: a norm before and one after every
     sublayer (the feed-forward may be absent).  The first norm of a sublayer writes the products' operand in the
     compute type; the sublayer writes its result to a buffer of the block; one kernel then norms that buffer and
-    adds it to the 32-bit stream (it takes a product's K pieces in place of the buffer).  The norms are
+    adds it to the 32-bit stream (it takes a product's K pieces in place of the buffer) and, in the same pass over
+    the row, forms the norm that reads the stream next: the feed-forward's first norm behind the mixer, the next
+    layer's first norm behind the feed-forward when that layer is of this kind (``entry_hint``).  The norms are
     root-mean-square norms with a gain."""
     takes_pending = False
-    takes_next_norm = False
+    takes_next_norm = True
+    _READY = "sandwich_norm.operand"      # in step.memo: (stream, gain, operand) of a norm that the kernel before formed
 
     def __init__(self, spec: BlockSpec, ctx: BuildContext):
         if spec.mixer_out_norm is None or (spec.ffn is not None and (spec.ffn_norm is None or spec.ffn_out_norm is None)):
@@ -357,29 +360,55 @@ class SandwichNormBlock(Part):
         return n_tokens * self.hidden * (size + 4) + self.mixer.activation_bytes(n_tokens) + \
             (self.ffn.activation_bytes(n_tokens) if self.ffn is not None else 0)
 
-    def _sublayer(self, step, x, norm, run, out_norm) -> None:
+    def entry_hint(self, step):
+        """The norm this block reads the stream with first, for the kernel that completes the stream before it."""
+        norm = self.children["mixer_norm"]
+        gain = getattr(norm, "gain", None)
+        if gain is None or not hasattr(norm, "eps") or getattr(norm, "centred", False):
+            return None
+        return FullNormHint(gain, float(norm.eps), self.hidden)
+
+    def _sublayer(self, step, x, norm, run, out_norm, following) -> None:
+        """``following``: a ``FullNormHint`` of the norm that reads the stream after this sublayer, or None."""
         ws = step.workspace
         rs = stream(step)
-        xn = ws.get("block.xn", tuple(x.shape), self.dtype)
-        norm.forward(x, xn)
+        ready = step.memo.pop(self._READY, None)
+        gain = getattr(norm, "gain", None)
+        if ready is not None and gain is not None and ready[0] == x.data_ptr() and ready[1] == gain.data_ptr():
+            xn = ready[2]           # the kernel that completed the stream formed this norm on its way
+        else:
+            xn = ws.get("block.xn", tuple(x.shape), self.dtype)
+            norm.forward(x, xn)
         y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
         rs.overwrite = rs.defer_overwrite = True
         run(xn, y)
         # (a product cut along K may have left its pieces for this kernel to add: they are all of y then)
         pending = ws.take_pending_or_whole(y)
         partials, replace = pending if pending is not None else (None, False)
-        ops.norm_add(x, y, out_norm.gain, None, out_norm.eps, layer=False, partials=partials, replace=replace)
+        if isinstance(following, FullNormHint) and following.width == x.shape[1]:
+            # (the sublayer is done with its operand: the buffer takes the next one)
+            nxt = ws.get("block.xn", tuple(x.shape), self.dtype)
+            ops.norm_add(x, y, out_norm.gain, None, out_norm.eps, layer=False, partials=partials, replace=replace, copy=nxt,
+                         next_gain=following.gain, next_eps=following.eps)
+            step.memo[self._READY] = (x.data_ptr(), following.gain.data_ptr(), nxt)
+        else:
+            ops.norm_add(x, y, out_norm.gain, None, out_norm.eps, layer=False, partials=partials, replace=replace)
 
-    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool, next_norm=None) -> None:
         rs = stream(step)
         step.workspace.flush_pending()
         rs.row_scale = rs.next_norm = None
         try:
+            inner = None
+            if self.ffn is not None:
+                n2 = self.children["ffn_norm"]
+                if getattr(n2, "gain", None) is not None and hasattr(n2, "eps") and not getattr(n2, "centred", False):
+                    inner = FullNormHint(n2.gain, float(n2.eps), self.hidden)
             self._sublayer(step, x, self.children["mixer_norm"], lambda xn, y: self.mixer.forward(step, xn, y, cache, owns_cache),
-                           self.children["mixer_out_norm"])
+                           self.children["mixer_out_norm"], inner if self.ffn is not None else next_norm)
             if self.ffn is not None:
                 self._sublayer(step, x, self.children["ffn_norm"], lambda xn, y: self.ffn.forward(step, xn, y),
-                               self.children["ffn_out_norm"])
+                               self.children["ffn_out_norm"], next_norm)
         finally:
             rs.overwrite = rs.defer_overwrite = False
 

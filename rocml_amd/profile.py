@@ -126,7 +126,8 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "sigmoid_gate": ("output gate", lambda y, gate, **kw: (2 * _nbytes(y) + gate.numel() * 4, 4 * y.numel())),
     "qk_span_stats": ("q/k norm factors", lambda qkv, q_width, k_width, bias, eps, out: (
         qkv.shape[0] * (q_width + k_width) * qkv.element_size() + _nbytes(out), 2 * qkv.shape[0] * (q_width + k_width))),
-    "norm_add": ("sublayer norm and residual sum", lambda x, y, gain, bias, eps, **kw: (
+    "norm_add": (lambda *a, **kw: "sublayer norm, residual sum and the next norm" if kw.get("next_gain") is not None
+                 else "sublayer norm and residual sum", lambda x, y, gain, bias, eps, **kw: (
         2 * _nbytes(x) + _nbytes(kw.get("copy"), kw.get("partials")) + (0 if kw.get("replace") else _nbytes(y)), 8 * x.numel())),
     "norm_add_branches": ("branch norms, sublayer norm and residual sum", lambda x, branches, gains, weight, beps, gain, bias, eps, layer, **kw: (
         2 * _nbytes(x) + _nbytes(*branches) + _nbytes(kw.get("copy")), 8 * x.numel() * (1 + len(branches)))),

@@ -323,3 +323,26 @@ def test_small_sums_and_the_soft_cap():
     want = 12.0 * torch.tanh(z.cpu().double() / 12.0)
     ops.softcap(z, 12.0)
     _close(z, want, 1e-6, "soft cap")
+
+
+@pytest.mark.parametrize("n", [5, 36, 70, 72, 1024, 4100])
+def test_sublayer_norm_with_the_next_norm(n):
+    """The kernel that norms a sublayer's output and adds it to the stream also forms the norm that reads the stream next,
+    with and without the pieces of a product in place of the sublayer's output."""
+    from rocml_amd import ops
+    g = _gen(n)
+    rows, eps, eps2 = 6, 1e-5, 1e-3
+    x, y = torch.randn(rows, n, generator=g) * 3, torch.randn(rows, n, generator=g) * 5
+    parts = torch.randn(2, rows, n, generator=g)
+    w, w2 = 0.3 * torch.randn(n, generator=g), 0.3 * torch.randn(n, generator=g)
+    for with_parts in (False, True):
+        total = y.double() + (parts.double().sum(0) if with_parts else 0)
+        new_x = x.double() + plain.offset_norm(total, w.double(), eps)
+        want_next = plain.offset_norm(new_x, w2.double(), eps2)
+        for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+            xs = x.clone().to(DEV)
+            nxt = torch.empty(rows, n, dtype=dtype, device=DEV)
+            ops.norm_add(xs, y.clone().to(DEV), (1 + w).to(DEV), None, eps, layer=False, copy=nxt, partials=parts.to(DEV) if with_parts else None,
+                         next_gain=(1 + w2).to(DEV), next_eps=eps2)
+            _close(xs, new_x, 1e-5, "stream")
+            _close(nxt, want_next, tol, "the next norm")
