@@ -157,7 +157,7 @@ def roravik_config(vocab, width, heads, kv_heads, dim, window, ret_heads, ret_di
     retention in the odd ones; a dense feed-forward and routed experts (two groups of which one is kept, and a shared
     expert of twice an expert's size) in turn.  ``loop``: ``(start, stop, times)`` or None."""
     rot = {"base": 10000.0, "dims": dim}
-    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": conv, "scale": dim ** -0.5, "softcap": 30.0,
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": conv, "scale": dim ** -0.5, "softcap": 50.0,
             "mask": {"size": window}, "rot": rot}
     right = {"heads": mix_heads, "dim": mix_dim, "decay_rank": decay_rank}
     decay = [1.0 - 2.0 ** (-5 - 6 * h / max(ret_heads - 1, 1)) for h in range(ret_heads)]
@@ -173,7 +173,7 @@ def roravik_config(vocab, width, heads, kv_heads, dim, window, ret_heads, ret_di
         else:
             layers.append({"type": "retention", "mixer": retention, "mlp": mlp})
     cfg = {"architecture": "Roravik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": width ** 0.5},
-           "logit_softcap": 30.0, "layers": layers}
+           "logit_softcap": 25.0, "layers": layers}
     if loop is not None:
         cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
     return cfg
@@ -182,7 +182,7 @@ def roravik_config(vocab, width, heads, kv_heads, dim, window, ret_heads, ret_di
 # The fifth architecture: a test-sized model and the layer sizes of a 2B-class model (random weights; no
 # checkpoint of this design exists).
 CATALOG += [
-    ModelEntry("roravik-tiny", roravik_config(320, 96, 4, 2, 32, 40, 2, 24, 2, 16, 160, 8, 48, 2, 4, loop=(0, 2, 2), decay_rank=8),
+    ModelEntry("roravik-tiny", roravik_config(352, 96, 4, 2, 32, 48, 2, 24, 2, 16, 160, 8, 48, 2, 4, loop=(0, 2, 2), decay_rank=8),
                default_ctx=512, init_norm_jitter=True),
     ModelEntry("roravik-2b", roravik_config(32768, 2048, 16, 8, 128, 1024, 16, 128, 32, 64, 6144, 32, 1024, 4, 24)),
 ]
