@@ -204,7 +204,9 @@ def _attend(q, k, v, dtype, scale, cap, window, sink, decode_from, perm_seed):
 
 
 @pytest.mark.parametrize("dtype,H,G,d,dv", [(torch.float32, 4, 2, 24, 16), (torch.float32, 2, 2, 64, 64), (torch.bfloat16, 4, 2, 64, 64),
-                                            (torch.bfloat16, 8, 1, 128, 128), (torch.bfloat16, 3, 3, 16, 40)])
+                                            (torch.bfloat16, 8, 1, 128, 128), (torch.bfloat16, 3, 3, 16, 40), (torch.bfloat16, 6, 2, 96, 96),
+                                            (torch.bfloat16, 2, 1, 256, 256), (torch.bfloat16, 4, 4, 32, 32), (torch.bfloat16, 4, 2, 192, 192),
+                                            (torch.bfloat16, 34, 2, 64, 64)])
 @pytest.mark.parametrize("window", [1, 5, 64, 65, 130])
 def test_window_edge_under_a_soft_cap_and_a_sink(dtype, H, G, d, dv, window):
     """One key is made to win by far: just inside the window it takes the whole output, just outside it nothing of it shows,
